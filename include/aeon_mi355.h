@@ -1,0 +1,170 @@
+/*
+ * C ABI of the MI355X (gfx950, wave64) routed-expert hot path for project-aeon.
+ *
+ * Every entry point is what the reference's own C++ entry point for the same step would bind
+ * (the file:line each one replaces is cited beside it; paths are relative to the reference
+ * tree). Conventions, which are the reference's (src/infrastructure/hip_check.hpp:19-27,
+ * aeon_w4a16_swizzled_gemv.hpp:176-181):
+ *   - plain pointers and sizes only; every `const void*`/`void*` named `d_…` is a DEVICE
+ *     pointer owned by the caller; `half` data is IEEE fp16 bits;
+ *   - device work is enqueued asynchronously on `stream` (a hipStream_t passed as void*,
+ *     NULL = the default stream) and nothing synchronizes unless stated;
+ *   - the return value is AEON_OK or an AEON_ERR_* code, and aeon_last_error() returns the
+ *     calling thread's message. The C++ shims re-throw the reference's exception types:
+ *     AEON_ERR_INVALID_ARGUMENT -> std::invalid_argument, AEON_ERR_LOGIC -> std::logic_error,
+ *     AEON_ERR_OUT_OF_RANGE -> std::out_of_range, AEON_ERR_HIP -> std::runtime_error;
+ *   - nothing is thread-safe beyond the error string: one host thread drives one stream.
+ */
+#ifndef AEON_MI355_H
+#define AEON_MI355_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AEON_OK 0
+#define AEON_ERR_INVALID_ARGUMENT 1
+#define AEON_ERR_LOGIC 2
+#define AEON_ERR_OUT_OF_RANGE 3
+#define AEON_ERR_HIP 4
+
+const char* aeon_last_error(void);
+/* ABI revision of this header. */
+int aeon_abi_version(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Weight layout (host side, load time)
+ * ---------------------------------------------------------------------------------------- */
+
+/* aeon::swizzle_w4a16 / aeon::unswizzle_w4a16,
+ * src/backend/swizzled_w4a16/kernels/aeon_w4a16_swizzle.hpp:45-127, for 2-byte scales.
+ * Source layout: packed [N][K/8] u32 with column k in nibble k%8; scales [N][K/32].
+ * (rpw, lpr) is the reference SwizzleCfg: (4,8) for W1/W3, (8,4) for W2. Host pointers. */
+int aeon_swizzle_w4a16(const uint32_t* src_packed, const uint16_t* src_scale,
+                       uint32_t* dst_packed, uint16_t* dst_scale, int N, int K, int rpw, int lpr);
+int aeon_unswizzle_w4a16(const uint32_t* src_packed, const uint16_t* src_scale,
+                         uint32_t* dst_packed, uint16_t* dst_scale, int N, int K, int rpw, int lpr);
+
+/* The gfx950 wave64 packing ("A64"), the load-time re-swizzle of the `.aeon` payload
+ * (src/backend/swizzled_w4a16/core/swizzled_expert_format.hpp:9-30 is the layout it reads).
+ * A tile is 16 rows x 128 columns = 64 lanes x 16 bytes, tiles ordered [row/16][column/128];
+ * lane l holds row l%16 and, in word s of its uint4, columns 128g+32s+8(l/16)+0..7 in the
+ * payload's own nibble order; one fp16 scale per (row, 128-column group) at [tile][row%16].
+ * Requires N%16==0, K%128==0. Sizes in bytes: */
+size_t aeon_a64_packed_bytes(int N, int K);
+size_t aeon_a64_scale_bytes(int N, int K);
+/* Host repack of one swizzled matrix. Fails with AEON_ERR_INVALID_ARGUMENT when the four
+ * group-32 scales of any 128-group are not bit-equal (the layout stores one). */
+int aeon_a64_repack_host(const uint32_t* swz_packed, const uint16_t* swz_scale, int N, int K,
+                         int rpw, int lpr, uint32_t* a64_packed, uint16_t* a64_scale);
+int aeon_a64_unrepack_host(const uint32_t* a64_packed, const uint16_t* a64_scale, int N, int K,
+                           int rpw, int lpr, uint32_t* swz_packed, uint16_t* swz_scale);
+/* Device repack (one launch). `d_mismatch` (int, nullable) is incremented once per 128-group
+ * whose four group-32 scales differ; the caller zeroes and reads it. */
+int aeon_a64_repack_device(const void* d_swz_packed, const void* d_swz_scale, int N, int K,
+                           int rpw, int lpr, void* d_a64_packed, void* d_a64_scale,
+                           int* d_mismatch, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Decode kernels over the `.aeon` swizzled layout (the drop-in entry points)
+ * ---------------------------------------------------------------------------------------- */
+
+/* dispatch_aeon_w4a16_swizzled_gemv<WAVES,RPW,LPR,ITERS>,
+ * src/backend/swizzled_w4a16/kernels/aeon_w4a16_swizzled_gemv.hpp:166-190.
+ * y[row] = sum_g scale[row,g] * dot(q[row,g,:]-8, x[32g..]); fp32 accumulate, fp16 out.
+ * The template arguments become runtime ints; K must equal iters*lpr*32 and N%rpw==0. */
+int aeon_w4a16_swizzled_gemv(const void* d_activation, const void* d_packed, const void* d_scale,
+                             void* d_output, int N, int K, int rpw, int lpr, void* stream);
+/* dispatch_aeon_w4a16_swizzled_dual_gemv, aeon_w4a16_swizzled_gemv.hpp:192-222. */
+int aeon_w4a16_swizzled_dual_gemv(const void* d_activation, const void* d_packed_a,
+                                  const void* d_scale_a, const void* d_packed_b,
+                                  const void* d_scale_b, void* d_output_a, void* d_output_b,
+                                  int N, int K, int rpw, int lpr, void* stream);
+
+#define AEON_SWIZZLED_MAX_EXPERTS 8
+/* SwizzledW13ExpertPtrs / SwizzledW2ExpertPtrs, aeon_moe_fused_w13.hpp:13-20 and
+ * aeon_moe_fused_w2.hpp:12-15: by-value tables of device pointers, same member order. */
+typedef struct {
+    const void* w1[AEON_SWIZZLED_MAX_EXPERTS];
+    const void* s1[AEON_SWIZZLED_MAX_EXPERTS];
+    const void* w3[AEON_SWIZZLED_MAX_EXPERTS];
+    const void* s3[AEON_SWIZZLED_MAX_EXPERTS];
+} aeon_w13_table;
+typedef struct {
+    const void* w2[AEON_SWIZZLED_MAX_EXPERTS];
+    const void* s2[AEON_SWIZZLED_MAX_EXPERTS];
+} aeon_w2_table;
+
+/* dispatch_dsv4_moe_gemv_w13_swiglu (src/architecture/deepseek_v4/kernels/
+ * moe_gemv_dispatch.hpp:28-45) = dispatch_aeon_moe_fused_gate_up with
+ * Dsv4ClampedSwiGLUEpilogue (aeon_moe_fused_w13.hpp:113-141, moe_grouped_epilogue.hpp:29-37):
+ * expert_hidden[e*N+row] = half(silu(min(g,L)) * clamp(u,-L,L)). `d_output_f32` (nullable) is
+ * zeroed for `output_dim` floats, as the reference kernel does (:55-61). */
+int aeon_moe_gemv_w13_swiglu(const void* d_activation, const aeon_w13_table* weights,
+                             void* d_expert_hidden, float* d_output_f32, int output_dim,
+                             int expert_count, int N, int K, int rpw, int lpr, float swiglu_limit,
+                             void* stream);
+/* dispatch_aeon_moe_fused_w2_contrib, aeon_moe_fused_w2.hpp:231-256:
+ * contrib[e*N+row] = topk_w[e] * (W2_e . hidden_e)[row], one writer per element. */
+int aeon_moe_fused_w2_contrib(const void* d_expert_hidden, const aeon_w2_table* weights,
+                              const float* d_topk_weights, float* d_contrib, int expert_count,
+                              int N, int K, int rpw, int lpr, void* stream);
+/* moe_accumulate_fixed_order_kernel launch, src/platform/ops/moe_accumulate.hpp:73-92:
+ * out[i] = half(float(shared[i]) + sum_{e ascending} contrib[e*hidden+i]); `d_shared` may be
+ * NULL and may alias `d_out`. */
+int aeon_moe_accumulate_fixed_order(const float* d_contrib, int expert_count,
+                                    const void* d_shared, void* d_out, int hidden, void* stream);
+/* v4_swiglu_clamp_kernel launch, src/architecture/deepseek_v4/kernels/v4_swiglu_clamp.hpp:18-34. */
+int aeon_swiglu_clamp(const void* d_gate, const void* d_up, void* d_out, int total_elements,
+                      float limit, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Decode kernels over the wave64 packing (the MI355X-native path)
+ * ---------------------------------------------------------------------------------------- */
+
+/* W4A16 GEMV over an A64 matrix: same arithmetic contract as
+ * dispatch_aeon_w4a16_swizzled_gemv (aeon_w4a16_swizzled_gemv.hpp:43-93,166-190) with one
+ * scale per 128 columns. VALU only (no MFMA): 1 KiB coalesced wave loads, in-register nibble
+ * dequant, K split across the waves of a workgroup and reduced by wave shuffles.
+ * `tokens` activations [tokens][K] (row pitch x_stride elements) give [tokens][N] outputs
+ * (pitch out_stride); 1 <= tokens <= 8. */
+int aeon_a64_gemv(const void* d_x, int x_stride, const void* d_packed, const void* d_scale,
+                  void* d_out, int out_stride, int tokens, int N, int K, void* stream);
+/* dispatch_aeon_w4a16_swizzled_dual_gemv (aeon_w4a16_swizzled_gemv.hpp:95-164,192-222) on A64:
+ * two matrices, one activation read. */
+int aeon_a64_dual_gemv(const void* d_x, int x_stride, const void* d_packed_a,
+                       const void* d_scale_a, const void* d_packed_b, const void* d_scale_b,
+                       void* d_out_a, void* d_out_b, int out_stride, int tokens, int N, int K,
+                       void* stream);
+
+/* One expert's six A64 sub-tensors (device pointers): the wave64 counterpart of the slot
+ * views UnifiedVRAMExpertPool::get_w{1,2,3}_{packed,scale} return
+ * (src/backend/swizzled_w4a16/core/vram_expert_pool.hpp:22-82). W1/W3 are [I][H], W2 [H][I]. */
+typedef struct {
+    const void* w1_packed;
+    const void* w1_scale;
+    const void* w3_packed;
+    const void* w3_scale;
+    const void* w2_packed;
+    const void* w2_scale;
+} aeon_a64_expert;
+
+/* One routed expert over `tokens` (1..16) activations [tokens][H]: the per-token trio of
+ * V4TieredExpertExecutor::accumulate_routed (src/architecture/deepseek_v4/moe/
+ * v4_expert_executor.hpp:298-370) for a single slot -- fused gate+up dual-GEMV with the
+ * clamped SwiGLU (hidden fp16 [tokens][I] into d_hidden), W2 with the routing weight
+ * (contrib fp32 [tokens][H] into d_contrib = w[t]*acc), then the fixed-order reduce with one
+ * slot: out[t] = half(float(shared[t]) + contrib[t]); d_shared nullable, may alias d_out.
+ * use_mfma 0 = VALU GEMV kernels (tokens <= 8), 1 = the MFMA segment kernels. */
+int aeon_a64_expert_decode(const void* d_x, int tokens, const aeon_a64_expert* expert,
+                           const float* d_route_weights, void* d_hidden, float* d_contrib,
+                           const void* d_shared, void* d_out, int H, int I, float swiglu_limit,
+                           int use_mfma, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,327 @@
+// Decode kernels that read the `.aeon` swizzled payload in place (no repack), so they can sit
+// behind the reference's own entry points whatever the caller does with its expert slots.
+//
+// The payload stores, per (row block, iteration), 32 uint4 = 512 contiguous bytes: lane
+// row_in_block*LPR + slice holds the 32 columns of group iteration*LPR + slice. A wave64 takes
+// two consecutive iterations at once, so each wave load is 1 KiB contiguous and each scale
+// load 128 B contiguous. A workgroup owns one row block; its waves split K (iterations)
+// between them, every lane keeps all of its loads in flight, and partial sums meet through a
+// wave xor-butterfly and a small LDS exchange. Bandwidth-bound by design: no MFMA.
+#include "common.hpp"
+
+namespace aeon355 {
+
+constexpr int kWaves = 4;            // waves per workgroup = K splits
+constexpr int kMaxItersPerLane = 8;  // iterations one lane may own (K <= 8*kWaves*2*LPR*32)
+
+enum class SwzMode { Gemv, Dual, GateUp, W2Contrib };
+
+struct SwzArgs {
+    const uint16_t* activation;  // fp16 bits
+    aeon_w13_table w13;          // GateUp (w1/s1/w3/s3); Gemv/Dual use slot 0
+    aeon_w2_table w2;            // W2Contrib
+    const float* topk_weights;
+    uint16_t* out_a;  // Gemv/Dual output a, GateUp expert_hidden
+    uint16_t* out_b;  // Dual output b
+    float* out_f32;   // W2Contrib contrib; GateUp optional zero-fill target
+    int zero_dim;
+    int expert_count;
+    int N;
+    int iterations;
+    float limit;
+};
+
+// One 32-column group of one row: 4 packed words against 64 bytes of activation.
+__device__ __forceinline__ float group32_dot(const uint4& words, const uint4* x) {
+    float acc = 0.0f;
+    acc = dot8(words.x, x[0], acc);
+    acc = dot8(words.y, x[1], acc);
+    acc = dot8(words.z, x[2], acc);
+    acc = dot8(words.w, x[3], acc);
+    return acc;
+}
+
+template <int RPW, int LPR, SwzMode MODE>
+__global__ __launch_bounds__(kWaves * 64) void swizzled_decode_kernel(SwzArgs a) {
+    static_assert(RPW * LPR == 32, "RPW and LPR describe one 32-slot storage tile");
+    constexpr bool kTwo = (MODE == SwzMode::Dual || MODE == SwzMode::GateUp);
+
+    const int expert = blockIdx.y;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int half_id = lane >> 5;
+    const int lane32 = lane & 31;
+    const int row_block = blockIdx.x;
+    const int row_in_block = lane32 / LPR;
+    const int slice = lane32 % LPR;
+
+    if (MODE == SwzMode::GateUp && expert == 0 && a.out_f32 != nullptr) {
+        for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < a.zero_dim;
+             i += gridDim.x * blockDim.x) {
+            a.out_f32[i] = 0.0f;
+        }
+    }
+
+    const uint4* pa;
+    const uint16_t* sa;
+    const uint4* pb = nullptr;
+    const uint16_t* sb = nullptr;
+    const uint16_t* x = a.activation;
+    if (MODE == SwzMode::W2Contrib) {
+        pa = static_cast<const uint4*>(a.w2.w2[expert]);
+        sa = static_cast<const uint16_t*>(a.w2.s2[expert]);
+        x += static_cast<size_t>(expert) * (static_cast<size_t>(a.iterations) * LPR * 32);
+    } else {
+        pa = static_cast<const uint4*>(a.w13.w1[expert]);
+        sa = static_cast<const uint16_t*>(a.w13.s1[expert]);
+        if (kTwo) {
+            pb = static_cast<const uint4*>(a.w13.w3[expert]);
+            sb = static_cast<const uint16_t*>(a.w13.s3[expert]);
+        }
+    }
+
+    // Iterations owned by this lane: 2*wave + half_id, stepping by 2*kWaves.
+    const size_t block_base = static_cast<size_t>(row_block) * a.iterations * 32 + lane32;
+    uint4 wa[kMaxItersPerLane], wb[kMaxItersPerLane];
+    uint16_t ca[kMaxItersPerLane], cb[kMaxItersPerLane];
+#pragma unroll
+    for (int j = 0; j < kMaxItersPerLane; ++j) {
+        const int it = 2 * wave + half_id + j * 2 * kWaves;
+        if (it < a.iterations) {
+            const size_t slot = block_base + static_cast<size_t>(it) * 32;
+            wa[j] = pa[slot];
+            ca[j] = sa[slot];
+            if (kTwo) {
+                wb[j] = pb[slot];
+                cb[j] = sb[slot];
+            }
+        }
+    }
+
+    float acc_a = 0.0f, acc_b = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kMaxItersPerLane; ++j) {
+        const int it = 2 * wave + half_id + j * 2 * kWaves;
+        if (it < a.iterations) {
+            const int group = it * LPR + slice;
+            const uint4* xg = reinterpret_cast<const uint4*>(x + static_cast<size_t>(group) * 32);
+            uint4 xv[4] = {xg[0], xg[1], xg[2], xg[3]};
+            acc_a += half_bits_to_float(ca[j]) * group32_dot(wa[j], xv);
+            if (kTwo) acc_b += half_bits_to_float(cb[j]) * group32_dot(wb[j], xv);
+        }
+    }
+
+    // Lanes of one row: the LPR slices (low bits of lane32) and the two halves (bit 5).
+    acc_a = wave_xor_sum(acc_a, (LPR - 1) | 32);
+    if (kTwo) acc_b = wave_xor_sum(acc_b, (LPR - 1) | 32);
+
+    __shared__ float partial[2][kWaves][RPW];
+    if (half_id == 0 && slice == 0) {
+        partial[0][wave][row_in_block] = acc_a;
+        if (kTwo) partial[1][wave][row_in_block] = acc_b;
+    }
+    __syncthreads();
+
+    if (threadIdx.x < RPW) {
+        const int row = row_block * RPW + threadIdx.x;
+        float sum_a = 0.0f, sum_b = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            sum_a += partial[0][w][threadIdx.x];
+            if (kTwo) sum_b += partial[1][w][threadIdx.x];
+        }
+        if (row < a.N) {
+            if (MODE == SwzMode::Gemv) {
+                a.out_a[row] = float_to_half_bits(sum_a);
+            } else if (MODE == SwzMode::Dual) {
+                a.out_a[row] = float_to_half_bits(sum_a);
+                a.out_b[row] = float_to_half_bits(sum_b);
+            } else if (MODE == SwzMode::GateUp) {
+                a.out_a[static_cast<size_t>(expert) * a.N + row] =
+                    float_to_half_bits(clamped_swiglu(sum_a, sum_b, a.limit));
+            } else {
+                a.out_f32[static_cast<size_t>(expert) * a.N + row] = a.topk_weights[expert] * sum_a;
+            }
+        }
+    }
+}
+
+template <SwzMode MODE>
+static int launch(const SwzArgs& a, int rpw, int lpr, int experts, hipStream_t stream,
+                  const char* who) {
+    const dim3 block(kWaves * 64);
+    if (rpw == 4 && lpr == 8) {
+        swizzled_decode_kernel<4, 8, MODE><<<dim3(a.N / 4, experts), block, 0, stream>>>(a);
+    } else if (rpw == 8 && lpr == 4) {
+        swizzled_decode_kernel<8, 4, MODE><<<dim3(a.N / 8, experts), block, 0, stream>>>(a);
+    } else if (rpw == 2 && lpr == 16) {
+        swizzled_decode_kernel<2, 16, MODE><<<dim3(a.N / 2, experts), block, 0, stream>>>(a);
+    } else if (rpw == 16 && lpr == 2) {
+        swizzled_decode_kernel<16, 2, MODE><<<dim3(a.N / 16, experts), block, 0, stream>>>(a);
+    } else {
+        set_error("%s: unsupported swizzle geometry rpw=%d lpr=%d", who, rpw, lpr);
+        return AEON_ERR_INVALID_ARGUMENT;
+    }
+    AEON_LAUNCH_CHECK();
+    return AEON_OK;
+}
+
+// The reference dispatchers' shape rule (aeon_w4a16_swizzled_gemv.hpp:176-181) with the
+// template arguments as runtime values, plus this kernel's own capacity.
+static int check_shape(int N, int K, int rpw, int lpr, const char* who) {
+    AEON_REQUIRE(rpw > 0 && lpr > 0 && rpw * lpr == 32, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: rpw*lpr must be 32 (rpw=%d lpr=%d)", who, rpw, lpr);
+    AEON_REQUIRE(N > 0 && K > 0 && K % (lpr * 32) == 0 && N % rpw == 0, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: incompatible N/K shape (N=%d K=%d rpw=%d lpr=%d)", who, N, K, rpw, lpr);
+    AEON_REQUIRE(K / (lpr * 32) <= kMaxItersPerLane * 2 * kWaves, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: K=%d exceeds the kernel's capacity of %d columns at lpr=%d", who, K,
+                 kMaxItersPerLane * 2 * kWaves * lpr * 32, lpr);
+    return AEON_OK;
+}
+
+__global__ __launch_bounds__(256) void accumulate_fixed_order_kernel(
+    const float* __restrict__ contrib, int expert_count, const uint16_t* shared, uint16_t* out,
+    int hidden) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= hidden) return;
+    float acc = shared != nullptr ? half_bits_to_float(shared[i]) : 0.0f;
+    for (int e = 0; e < expert_count; ++e) acc += contrib[static_cast<size_t>(e) * hidden + i];
+    out[i] = float_to_half_bits(acc);
+}
+
+__global__ __launch_bounds__(256) void swiglu_clamp_kernel(const uint16_t* __restrict__ gate,
+                                                           const uint16_t* __restrict__ up,
+                                                           uint16_t* __restrict__ out, int total,
+                                                           float limit) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < total) {
+        out[i] = float_to_half_bits(
+            clamped_swiglu(half_bits_to_float(gate[i]), half_bits_to_float(up[i]), limit));
+    }
+}
+
+}  // namespace aeon355
+
+using namespace aeon355;
+
+extern "C" int aeon_w4a16_swizzled_gemv(const void* d_activation, const void* d_packed,
+                                        const void* d_scale, void* d_output, int N, int K, int rpw,
+                                        int lpr, void* stream) {
+    const char* who = "aeon_w4a16_swizzled_gemv";
+    AEON_REQUIRE(d_activation && d_packed && d_scale && d_output, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: null buffer", who);
+    if (int rc = check_shape(N, K, rpw, lpr, who)) return rc;
+    SwzArgs a{};
+    a.activation = static_cast<const uint16_t*>(d_activation);
+    a.w13.w1[0] = d_packed;
+    a.w13.s1[0] = d_scale;
+    a.out_a = static_cast<uint16_t*>(d_output);
+    a.N = N;
+    a.iterations = K / (lpr * 32);
+    return launch<SwzMode::Gemv>(a, rpw, lpr, 1, as_stream(stream), who);
+}
+
+extern "C" int aeon_w4a16_swizzled_dual_gemv(const void* d_activation, const void* d_packed_a,
+                                             const void* d_scale_a, const void* d_packed_b,
+                                             const void* d_scale_b, void* d_output_a,
+                                             void* d_output_b, int N, int K, int rpw, int lpr,
+                                             void* stream) {
+    const char* who = "aeon_w4a16_swizzled_dual_gemv";
+    AEON_REQUIRE(d_activation && d_packed_a && d_scale_a && d_packed_b && d_scale_b &&
+                     d_output_a && d_output_b,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
+    if (int rc = check_shape(N, K, rpw, lpr, who)) return rc;
+    SwzArgs a{};
+    a.activation = static_cast<const uint16_t*>(d_activation);
+    a.w13.w1[0] = d_packed_a;
+    a.w13.s1[0] = d_scale_a;
+    a.w13.w3[0] = d_packed_b;
+    a.w13.s3[0] = d_scale_b;
+    a.out_a = static_cast<uint16_t*>(d_output_a);
+    a.out_b = static_cast<uint16_t*>(d_output_b);
+    a.N = N;
+    a.iterations = K / (lpr * 32);
+    return launch<SwzMode::Dual>(a, rpw, lpr, 1, as_stream(stream), who);
+}
+
+extern "C" int aeon_moe_gemv_w13_swiglu(const void* d_activation, const aeon_w13_table* weights,
+                                        void* d_expert_hidden, float* d_output_f32, int output_dim,
+                                        int expert_count, int N, int K, int rpw, int lpr,
+                                        float swiglu_limit, void* stream) {
+    const char* who = "aeon_moe_gemv_w13_swiglu";
+    AEON_REQUIRE(d_activation && weights && d_expert_hidden, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: null buffer", who);
+    AEON_REQUIRE(expert_count > 0 && expert_count <= AEON_SWIZZLED_MAX_EXPERTS,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: expert_count %d outside 1..%d", who, expert_count,
+                 AEON_SWIZZLED_MAX_EXPERTS);
+    if (int rc = check_shape(N, K, rpw, lpr, who)) return rc;
+    for (int e = 0; e < expert_count; ++e) {
+        AEON_REQUIRE(weights->w1[e] && weights->s1[e] && weights->w3[e] && weights->s3[e],
+                     AEON_ERR_INVALID_ARGUMENT, "%s: expert slot %d has a null weight pointer", who, e);
+    }
+    SwzArgs a{};
+    a.activation = static_cast<const uint16_t*>(d_activation);
+    a.w13 = *weights;
+    a.out_a = static_cast<uint16_t*>(d_expert_hidden);
+    a.out_f32 = d_output_f32;
+    a.zero_dim = output_dim;
+    a.expert_count = expert_count;
+    a.N = N;
+    a.iterations = K / (lpr * 32);
+    a.limit = swiglu_limit;
+    return launch<SwzMode::GateUp>(a, rpw, lpr, expert_count, as_stream(stream), who);
+}
+
+extern "C" int aeon_moe_fused_w2_contrib(const void* d_expert_hidden, const aeon_w2_table* weights,
+                                         const float* d_topk_weights, float* d_contrib,
+                                         int expert_count, int N, int K, int rpw, int lpr,
+                                         void* stream) {
+    const char* who = "aeon_moe_fused_w2_contrib";
+    AEON_REQUIRE(d_expert_hidden && weights && d_topk_weights && d_contrib,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
+    AEON_REQUIRE(expert_count > 0 && expert_count <= AEON_SWIZZLED_MAX_EXPERTS,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: expert_count %d outside 1..%d", who, expert_count,
+                 AEON_SWIZZLED_MAX_EXPERTS);
+    if (int rc = check_shape(N, K, rpw, lpr, who)) return rc;
+    for (int e = 0; e < expert_count; ++e) {
+        AEON_REQUIRE(weights->w2[e] && weights->s2[e], AEON_ERR_INVALID_ARGUMENT,
+                     "%s: expert slot %d has a null weight pointer", who, e);
+    }
+    SwzArgs a{};
+    a.activation = static_cast<const uint16_t*>(d_expert_hidden);
+    a.w2 = *weights;
+    a.topk_weights = d_topk_weights;
+    a.out_f32 = d_contrib;
+    a.expert_count = expert_count;
+    a.N = N;
+    a.iterations = K / (lpr * 32);
+    return launch<SwzMode::W2Contrib>(a, rpw, lpr, expert_count, as_stream(stream), who);
+}
+
+extern "C" int aeon_moe_accumulate_fixed_order(const float* d_contrib, int expert_count,
+                                               const void* d_shared, void* d_out, int hidden,
+                                               void* stream) {
+    AEON_REQUIRE(d_contrib && d_out, AEON_ERR_INVALID_ARGUMENT,
+                 "aeon_moe_accumulate_fixed_order: null buffer");
+    AEON_REQUIRE(expert_count >= 0 && hidden > 0, AEON_ERR_INVALID_ARGUMENT,
+                 "aeon_moe_accumulate_fixed_order: bad shape (experts=%d hidden=%d)", expert_count,
+                 hidden);
+    accumulate_fixed_order_kernel<<<(hidden + 255) / 256, 256, 0, as_stream(stream)>>>(
+        d_contrib, expert_count, static_cast<const uint16_t*>(d_shared),
+        static_cast<uint16_t*>(d_out), hidden);
+    AEON_LAUNCH_CHECK();
+    return AEON_OK;
+}
+
+extern "C" int aeon_swiglu_clamp(const void* d_gate, const void* d_up, void* d_out,
+                                 int total_elements, float limit, void* stream) {
+    AEON_REQUIRE(d_gate && d_up && d_out, AEON_ERR_INVALID_ARGUMENT, "aeon_swiglu_clamp: null buffer");
+    AEON_REQUIRE(total_elements >= 0, AEON_ERR_INVALID_ARGUMENT,
+                 "aeon_swiglu_clamp: negative element count");
+    if (total_elements == 0) return AEON_OK;
+    swiglu_clamp_kernel<<<(total_elements + 255) / 256, 256, 0, as_stream(stream)>>>(
+        static_cast<const uint16_t*>(d_gate), static_cast<const uint16_t*>(d_up),
+        static_cast<uint16_t*>(d_out), total_elements, limit);
+    AEON_LAUNCH_CHECK();
+    return AEON_OK;
+}

@@ -1,0 +1,494 @@
+// Decode kernels over the wave64 ("A64") packing.
+//
+// Two families, both HBM-bound by construction (every weight byte is read once per segment in
+// 1 KiB coalesced wave loads, scales at one fp16 per 128 columns):
+//
+//   * a64_gemv_kernel: VALU only. Lane (row l%16, chunk l/16) dequantises its 32 nibbles in
+//     registers and feeds v_dot2_f32_f16 against four 16-byte activation chunks; the four
+//     chunk lanes of a row meet through a wave xor-butterfly, K splits across the waves of the
+//     workgroup meet through LDS. This is the GEMV / dual-GEMV of the decode path.
+//   * a64_seg_kernel: for an expert that serves up to 16 tokens of a batch. The same 1 KiB
+//     tile is, unchanged, the A operand of four v_mfma_f32_16x16x32_f16 steps whose B operand
+//     is the 16 token rows, so the weight stream is read once however many of the 16 tokens are
+//     live and the VALU work per byte does not grow with the token count. The scale is applied
+//     in fp32 to the per-group MFMA result, so dequantisation stays exact.
+#include "expert_a64.hpp"
+
+namespace aeon355 {
+
+// ---------------------------------------------------------------------------------------------
+// VALU GEMV
+// ---------------------------------------------------------------------------------------------
+
+constexpr int kGemvPrefetch = 4;  // weight tiles a lane keeps in flight
+
+struct GemvArgs {
+    const uint16_t* x;
+    long x_stride;
+    const uint4* pa;
+    const uint16_t* sa;
+    const uint4* pb;
+    const uint16_t* sb;
+    uint16_t* out_a;
+    uint16_t* out_b;
+    long out_stride;
+    int tokens;
+    int N;
+    int groups;  // K / 128
+    // epilogue: 0 = fp16 rows of each matrix; 1 = out_a = half(clamped_swiglu(a, b));
+    // 2 = out_f32[t][row] = tok_weight[t] * a (one writer per element)
+    int epilogue;
+    float limit;
+    const float* tok_weight;
+    float* out_f32;
+};
+
+template <int NMAT, int TOK, int WK>
+__global__ __launch_bounds__(WK * 64) void a64_gemv_kernel(GemvArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int r = lane & 15;
+    const int chunk = lane >> 4;
+    const int tile = blockIdx.x;
+    const size_t tile_base = static_cast<size_t>(tile) * a.groups;
+
+    float acc[NMAT][TOK];
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+        for (int t = 0; t < TOK; ++t) acc[m][t] = 0.0f;
+
+    for (int g0 = wave; g0 < a.groups; g0 += WK * kGemvPrefetch) {
+        uint4 wq[NMAT][kGemvPrefetch];
+        uint16_t sc[NMAT][kGemvPrefetch];
+#pragma unroll
+        for (int j = 0; j < kGemvPrefetch; ++j) {
+            const int g = g0 + j * WK;
+            if (g < a.groups) {
+                wq[0][j] = a.pa[(tile_base + g) * 64 + lane];
+                sc[0][j] = a.sa[(tile_base + g) * 16 + r];
+                if (NMAT == 2) {
+                    wq[1][j] = a.pb[(tile_base + g) * 64 + lane];
+                    sc[1][j] = a.sb[(tile_base + g) * 16 + r];
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kGemvPrefetch; ++j) {
+            const int g = g0 + j * WK;
+            if (g < a.groups) {
+#pragma unroll
+                for (int t = 0; t < TOK; ++t) {
+                    if (t < a.tokens) {
+                        const uint16_t* xp = a.x + t * a.x_stride + g * 128 + chunk * 8;
+                        const uint4 x0 = *reinterpret_cast<const uint4*>(xp);
+                        const uint4 x1 = *reinterpret_cast<const uint4*>(xp + 32);
+                        const uint4 x2 = *reinterpret_cast<const uint4*>(xp + 64);
+                        const uint4 x3 = *reinterpret_cast<const uint4*>(xp + 96);
+#pragma unroll
+                        for (int m = 0; m < NMAT; ++m) {
+                            float d = 0.0f;
+                            d = dot8(wq[m][j].x, x0, d);
+                            d = dot8(wq[m][j].y, x1, d);
+                            d = dot8(wq[m][j].z, x2, d);
+                            d = dot8(wq[m][j].w, x3, d);
+                            acc[m][t] += half_bits_to_float(sc[m][j]) * d;
+                        }
+                    }
+                }
+            }
+        }
+    }
+
+    __shared__ float partial[WK][NMAT][TOK][16];
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+        for (int t = 0; t < TOK; ++t) {
+            const float v = wave_xor_sum(acc[m][t], 16 | 32);
+            if (chunk == 0) partial[wave][m][t][r] = v;
+        }
+    __syncthreads();
+
+    for (int i = threadIdx.x; i < NMAT * TOK * 16; i += WK * 64) {
+        const int row = i & 15;
+        const int t = (i >> 4) % TOK;
+        const int m = (i >> 4) / TOK;
+        if (t < a.tokens) {
+            float sum = 0.0f;
+#pragma unroll
+            for (int w = 0; w < WK; ++w) sum += partial[w][m][t][row];
+            const size_t at = t * a.out_stride + tile * 16 + row;
+            if (a.epilogue == 0) {
+                uint16_t* out = m == 0 ? a.out_a : a.out_b;
+                out[at] = float_to_half_bits(sum);
+            } else if (a.epilogue == 1) {
+                if (m == 0) {
+                    float up = 0.0f;
+#pragma unroll
+                    for (int w = 0; w < WK; ++w) up += partial[w][NMAT - 1][t][row];
+                    a.out_a[at] = float_to_half_bits(clamped_swiglu(sum, up, a.limit));
+                }
+            } else {
+                a.out_f32[at] = a.tok_weight[t] * sum;
+            }
+        }
+    }
+}
+
+template <int NMAT, int TOK>
+static int launch_gemv_wk(const GemvArgs& a, int wk, hipStream_t stream) {
+    const dim3 grid(a.N / 16);
+    if (wk >= 16) {
+        a64_gemv_kernel<NMAT, TOK, 16><<<grid, 16 * 64, 0, stream>>>(a);
+    } else if (wk >= 8) {
+        a64_gemv_kernel<NMAT, TOK, 8><<<grid, 8 * 64, 0, stream>>>(a);
+    } else {
+        a64_gemv_kernel<NMAT, TOK, 4><<<grid, 4 * 64, 0, stream>>>(a);
+    }
+    AEON_LAUNCH_CHECK();
+    return AEON_OK;
+}
+
+template <int NMAT>
+static int launch_gemv(const GemvArgs& a, hipStream_t stream) {
+    // Enough waves to cover 256 CUs a few times over: split K further when N is small.
+    const int tiles = a.N / 16;
+    int wk = 4;
+    while (wk < 16 && tiles * wk < 2048 && a.groups >= 2 * wk) wk *= 2;
+    if (a.tokens == 1) return launch_gemv_wk<NMAT, 1>(a, wk, stream);
+    if (a.tokens == 2) return launch_gemv_wk<NMAT, 2>(a, wk, stream);
+    if (a.tokens <= 4) return launch_gemv_wk<NMAT, 4>(a, wk, stream);
+    return launch_gemv_wk<NMAT, 8>(a, wk > 8 ? 8 : wk, stream);
+}
+
+static int check_a64_shape(int N, int K, const char* who) {
+    AEON_REQUIRE(N > 0 && K > 0 && N % 16 == 0 && K % 128 == 0, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: the wave64 packing needs N%%16==0 and K%%128==0 (N=%d K=%d)", who, N, K);
+    return AEON_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// MFMA segment kernels
+// ---------------------------------------------------------------------------------------------
+
+__device__ __forceinline__ float4_t mfma_group(const uint4& wq, const half8_t xf[4]) {
+    float4_t t = {0.0f, 0.0f, 0.0f, 0.0f};
+    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(unpack8_vec(wq.x), xf[0], t, 0, 0, 0);
+    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(unpack8_vec(wq.y), xf[1], t, 0, 0, 0);
+    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(unpack8_vec(wq.z), xf[2], t, 0, 0, 0);
+    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(unpack8_vec(wq.w), xf[3], t, 0, 0, 0);
+    return t;
+}
+
+__device__ __forceinline__ void scale_add(float4_t& acc, const float4_t& t, uint2 scale_bits) {
+    acc[0] += half_bits_to_float(static_cast<uint16_t>(scale_bits.x & 0xFFFFu)) * t[0];
+    acc[1] += half_bits_to_float(static_cast<uint16_t>(scale_bits.x >> 16)) * t[1];
+    acc[2] += half_bits_to_float(static_cast<uint16_t>(scale_bits.y & 0xFFFFu)) * t[2];
+    acc[3] += half_bits_to_float(static_cast<uint16_t>(scale_bits.y >> 16)) * t[3];
+}
+
+constexpr int kSegPrefetch = 2;  // 128-column groups per wave per step
+
+// One workgroup = one (16-row tile, segment). Lane l supplies weight row l%16 / token l%16 and
+// the 8-column chunk l/16 of each 32-column MFMA step; it ends up holding output rows
+// 4*(l/16)..+3 of token l%16.
+template <bool GATE_UP, int WK>
+__global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegDownArgs dn) {
+    const SegmentList& seg = GATE_UP ? gu.seg : dn.seg;
+    const int s = blockIdx.y;
+    int first = 0;
+    int count = GATE_UP ? gu.direct_count : dn.direct_count;
+    aeon_a64_expert e = GATE_UP ? gu.direct_expert : dn.direct_expert;
+    if (seg.total != nullptr) {
+        if (s >= *seg.total) return;
+        first = seg.first[s];
+        count = seg.count[s];
+        e = (GATE_UP ? gu.experts : dn.experts)[seg.expert[s]];
+    }
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int n = lane & 15;
+    const int chunk = lane >> 4;
+    const int tile = blockIdx.x;
+
+    const int K = GATE_UP ? gu.H : dn.I;
+    const int groups = K / 128;
+    const uint4* pa = static_cast<const uint4*>(GATE_UP ? e.w1_packed : e.w2_packed);
+    const uint16_t* sa = static_cast<const uint16_t*>(GATE_UP ? e.w1_scale : e.w2_scale);
+    const uint4* pb = static_cast<const uint4*>(e.w3_packed);
+    const uint16_t* sb = static_cast<const uint16_t*>(e.w3_scale);
+
+    // A padded token column repeats the segment's last live position: always a valid row, and
+    // its products land in output columns the store below never writes.
+    const int position = first + (n < count ? n : count - 1);
+    const uint16_t* xrow;
+    if (GATE_UP) {
+        const long row = gu.row_index != nullptr ? gu.row_index[position] : position;
+        xrow = gu.x + row * gu.x_stride + chunk * 8;
+    } else {
+        xrow = dn.hidden + static_cast<size_t>(position) * dn.I + chunk * 8;
+    }
+
+    const size_t tile_base = static_cast<size_t>(tile) * groups;
+    float4_t acc_a = {0.0f, 0.0f, 0.0f, 0.0f};
+    float4_t acc_b = {0.0f, 0.0f, 0.0f, 0.0f};
+
+    for (int g0 = wave; g0 < groups; g0 += WK * kSegPrefetch) {
+        uint4 wa[kSegPrefetch], wb[kSegPrefetch];
+        uint2 ca[kSegPrefetch], cb[kSegPrefetch];
+        half8_t xf[kSegPrefetch][4];
+#pragma unroll
+        for (int j = 0; j < kSegPrefetch; ++j) {
+            const int g = g0 + j * WK;
+            if (g < groups) {
+                wa[j] = pa[(tile_base + g) * 64 + lane];
+                ca[j] = *reinterpret_cast<const uint2*>(sa + (tile_base + g) * 16 + chunk * 4);
+                if (GATE_UP) {
+                    wb[j] = pb[(tile_base + g) * 64 + lane];
+                    cb[j] = *reinterpret_cast<const uint2*>(sb + (tile_base + g) * 16 + chunk * 4);
+                }
+#pragma unroll
+                for (int st = 0; st < 4; ++st) {
+                    xf[j][st] = *reinterpret_cast<const half8_t*>(xrow + g * 128 + st * 32);
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kSegPrefetch; ++j) {
+            const int g = g0 + j * WK;
+            if (g < groups) {
+                scale_add(acc_a, mfma_group(wa[j], xf[j]), ca[j]);
+                if (GATE_UP) scale_add(acc_b, mfma_group(wb[j], xf[j]), cb[j]);
+            }
+        }
+    }
+
+    if (WK > 1) {
+        __shared__ float4_t partial[WK][2][64];
+        partial[wave][0][lane] = acc_a;
+        if (GATE_UP) partial[wave][1][lane] = acc_b;
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int w = 1; w < WK; ++w) {
+            acc_a += partial[w][0][lane];
+            if (GATE_UP) acc_b += partial[w][1][lane];
+        }
+    }
+
+    if (n >= count) return;
+    const int row0 = tile * 16 + chunk * 4;
+    if (GATE_UP) {
+        uint2 packed;
+        packed.x = float_to_half_bits(clamped_swiglu(acc_a[0], acc_b[0], gu.limit)) |
+                   (static_cast<uint32_t>(float_to_half_bits(
+                        clamped_swiglu(acc_a[1], acc_b[1], gu.limit))) << 16);
+        packed.y = float_to_half_bits(clamped_swiglu(acc_a[2], acc_b[2], gu.limit)) |
+                   (static_cast<uint32_t>(float_to_half_bits(
+                        clamped_swiglu(acc_a[3], acc_b[3], gu.limit))) << 16);
+        *reinterpret_cast<uint2*>(gu.hidden + static_cast<size_t>(first + n) * gu.I + row0) = packed;
+    } else {
+        const float w = dn.weight[first + n];
+        const float4_t v = {w * acc_a[0], w * acc_a[1], w * acc_a[2], w * acc_a[3]};
+        const size_t out_row = dn.out_row != nullptr ? dn.out_row[first + n] : first + n;
+        *reinterpret_cast<float4_t*>(dn.contrib + out_row * dn.H + row0) = v;
+    }
+}
+
+int launch_seg_gate_up(const SegGateUpArgs& a, int k_split, hipStream_t stream) {
+    AEON_REQUIRE(a.H % 128 == 0 && a.I % 16 == 0 && a.x_stride % 8 == 0, AEON_ERR_INVALID_ARGUMENT,
+                 "gate/up segments: need H%%128==0, I%%16==0 and an activation pitch that keeps "
+                 "rows 16-byte aligned (H=%d I=%d pitch=%ld)", a.H, a.I, a.x_stride);
+    if (a.seg.capacity <= 0) return AEON_OK;
+    const dim3 grid(a.I / 16, a.seg.capacity);
+    const SegDownArgs none{};
+    if (k_split >= 4) {
+        a64_seg_kernel<true, 4><<<grid, 256, 0, stream>>>(a, none);
+    } else if (k_split == 2) {
+        a64_seg_kernel<true, 2><<<grid, 128, 0, stream>>>(a, none);
+    } else {
+        a64_seg_kernel<true, 1><<<grid, 64, 0, stream>>>(a, none);
+    }
+    AEON_LAUNCH_CHECK();
+    return AEON_OK;
+}
+
+int launch_seg_down(const SegDownArgs& a, int k_split, hipStream_t stream) {
+    AEON_REQUIRE(a.I % 128 == 0 && a.H % 16 == 0, AEON_ERR_INVALID_ARGUMENT,
+                 "down segments: need I%%128==0 and H%%16==0 (H=%d I=%d)", a.H, a.I);
+    if (a.seg.capacity <= 0) return AEON_OK;
+    const dim3 grid(a.H / 16, a.seg.capacity);
+    const SegGateUpArgs none{};
+    if (k_split >= 4) {
+        a64_seg_kernel<false, 4><<<grid, 256, 0, stream>>>(none, a);
+    } else if (k_split == 2) {
+        a64_seg_kernel<false, 2><<<grid, 128, 0, stream>>>(none, a);
+    } else {
+        a64_seg_kernel<false, 1><<<grid, 64, 0, stream>>>(none, a);
+    }
+    AEON_LAUNCH_CHECK();
+    return AEON_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Fixed-order reduce over a token's slots
+// ---------------------------------------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void token_reduce_kernel(
+    const float* __restrict__ contrib, int slots, int shared_base, const uint16_t* initial,
+    long initial_stride, uint16_t* out, long out_stride, int hidden) {
+    const int t = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= hidden) return;
+    float acc = 0.0f;
+    if (shared_base >= 0) {
+        // The shared expert enters as an fp16 value, as it does when a separate pass has
+        // stored it into the token's accumulator first.
+        acc = half_bits_to_float(float_to_half_bits(
+            contrib[static_cast<size_t>(shared_base + t) * hidden + i]));
+    } else if (initial != nullptr) {
+        acc = half_bits_to_float(initial[t * initial_stride + i]);
+    }
+    const float* c = contrib + static_cast<size_t>(t) * slots * hidden + i;
+    for (int s = 0; s < slots; ++s) acc += c[static_cast<size_t>(s) * hidden];
+    out[t * out_stride + i] = float_to_half_bits(acc);
+}
+
+int launch_token_reduce(const float* contrib, int tokens, int slots, int shared_base,
+                        const uint16_t* initial, long initial_stride, uint16_t* out,
+                        long out_stride, int hidden, hipStream_t stream) {
+    if (tokens <= 0) return AEON_OK;
+    token_reduce_kernel<<<dim3((hidden + 255) / 256, tokens), 256, 0, stream>>>(
+        contrib, slots, shared_base, initial, initial_stride, out, out_stride, hidden);
+    AEON_LAUNCH_CHECK();
+    return AEON_OK;
+}
+
+}  // namespace aeon355
+
+using namespace aeon355;
+
+extern "C" int aeon_a64_gemv(const void* d_x, int x_stride, const void* d_packed,
+                             const void* d_scale, void* d_out, int out_stride, int tokens, int N,
+                             int K, void* stream) {
+    const char* who = "aeon_a64_gemv";
+    AEON_REQUIRE(d_x && d_packed && d_scale && d_out, AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
+    if (int rc = check_a64_shape(N, K, who)) return rc;
+    AEON_REQUIRE(tokens >= 1 && tokens <= 8, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: tokens=%d outside 1..8", who, tokens);
+    AEON_REQUIRE(x_stride >= K && x_stride % 8 == 0 && out_stride >= N, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: bad row pitch (x_stride=%d out_stride=%d)", who, x_stride, out_stride);
+    GemvArgs a{};
+    a.x = static_cast<const uint16_t*>(d_x);
+    a.x_stride = x_stride;
+    a.pa = static_cast<const uint4*>(d_packed);
+    a.sa = static_cast<const uint16_t*>(d_scale);
+    a.out_a = static_cast<uint16_t*>(d_out);
+    a.out_stride = out_stride;
+    a.tokens = tokens;
+    a.N = N;
+    a.groups = K / 128;
+    return launch_gemv<1>(a, as_stream(stream));
+}
+
+extern "C" int aeon_a64_dual_gemv(const void* d_x, int x_stride, const void* d_packed_a,
+                                  const void* d_scale_a, const void* d_packed_b,
+                                  const void* d_scale_b, void* d_out_a, void* d_out_b,
+                                  int out_stride, int tokens, int N, int K, void* stream) {
+    const char* who = "aeon_a64_dual_gemv";
+    AEON_REQUIRE(d_x && d_packed_a && d_scale_a && d_packed_b && d_scale_b && d_out_a && d_out_b,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
+    if (int rc = check_a64_shape(N, K, who)) return rc;
+    AEON_REQUIRE(tokens >= 1 && tokens <= 8, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: tokens=%d outside 1..8", who, tokens);
+    AEON_REQUIRE(x_stride >= K && x_stride % 8 == 0 && out_stride >= N, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: bad row pitch (x_stride=%d out_stride=%d)", who, x_stride, out_stride);
+    GemvArgs a{};
+    a.x = static_cast<const uint16_t*>(d_x);
+    a.x_stride = x_stride;
+    a.pa = static_cast<const uint4*>(d_packed_a);
+    a.sa = static_cast<const uint16_t*>(d_scale_a);
+    a.pb = static_cast<const uint4*>(d_packed_b);
+    a.sb = static_cast<const uint16_t*>(d_scale_b);
+    a.out_a = static_cast<uint16_t*>(d_out_a);
+    a.out_b = static_cast<uint16_t*>(d_out_b);
+    a.out_stride = out_stride;
+    a.tokens = tokens;
+    a.N = N;
+    a.groups = K / 128;
+    return launch_gemv<2>(a, as_stream(stream));
+}
+
+extern "C" int aeon_a64_expert_decode(const void* d_x, int tokens, const aeon_a64_expert* expert,
+                                      const float* d_route_weights, void* d_hidden,
+                                      float* d_contrib, const void* d_shared, void* d_out, int H,
+                                      int I, float swiglu_limit, int use_mfma, void* stream) {
+    const char* who = "aeon_a64_expert_decode";
+    AEON_REQUIRE(d_x && expert && d_route_weights && d_hidden && d_contrib && d_out,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
+    AEON_REQUIRE(expert->w1_packed && expert->w1_scale && expert->w3_packed && expert->w3_scale &&
+                     expert->w2_packed && expert->w2_scale,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: the expert has a null sub-tensor", who);
+    AEON_REQUIRE(H > 0 && I > 0 && H % 128 == 0 && I % 128 == 0, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: need H%%128==0 and I%%128==0 (H=%d I=%d)", who, H, I);
+    AEON_REQUIRE(tokens >= 1 && tokens <= (use_mfma ? kSegTokens : 8), AEON_ERR_INVALID_ARGUMENT,
+                 "%s: tokens=%d outside 1..%d for this kernel family", who, tokens,
+                 use_mfma ? kSegTokens : 8);
+    hipStream_t s = as_stream(stream);
+    if (use_mfma) {
+        SegGateUpArgs gu{};
+        gu.x = static_cast<const uint16_t*>(d_x);
+        gu.x_stride = H;
+        gu.hidden = static_cast<uint16_t*>(d_hidden);
+        gu.H = H;
+        gu.I = I;
+        gu.limit = swiglu_limit;
+        gu.seg.capacity = 1;
+        gu.direct_expert = *expert;
+        gu.direct_count = tokens;
+        if (int rc = launch_seg_gate_up(gu, 4, s)) return rc;
+        SegDownArgs dn{};
+        dn.hidden = static_cast<const uint16_t*>(d_hidden);
+        dn.weight = d_route_weights;
+        dn.contrib = d_contrib;
+        dn.H = H;
+        dn.I = I;
+        dn.seg.capacity = 1;
+        dn.direct_expert = *expert;
+        dn.direct_count = tokens;
+        if (int rc = launch_seg_down(dn, 4, s)) return rc;
+    } else {
+        GemvArgs g{};
+        g.x = static_cast<const uint16_t*>(d_x);
+        g.x_stride = H;
+        g.pa = static_cast<const uint4*>(expert->w1_packed);
+        g.sa = static_cast<const uint16_t*>(expert->w1_scale);
+        g.pb = static_cast<const uint4*>(expert->w3_packed);
+        g.sb = static_cast<const uint16_t*>(expert->w3_scale);
+        g.out_a = static_cast<uint16_t*>(d_hidden);
+        g.out_stride = I;
+        g.tokens = tokens;
+        g.N = I;
+        g.groups = H / 128;
+        g.epilogue = 1;
+        g.limit = swiglu_limit;
+        if (int rc = launch_gemv<2>(g, s)) return rc;
+        GemvArgs d{};
+        d.x = static_cast<const uint16_t*>(d_hidden);
+        d.x_stride = I;
+        d.pa = static_cast<const uint4*>(expert->w2_packed);
+        d.sa = static_cast<const uint16_t*>(expert->w2_scale);
+        d.out_f32 = d_contrib;
+        d.out_stride = H;
+        d.tokens = tokens;
+        d.N = H;
+        d.groups = I / 128;
+        d.epilogue = 2;
+        d.tok_weight = d_route_weights;
+        if (int rc = launch_gemv<1>(d, s)) return rc;
+    }
+    return launch_token_reduce(d_contrib, tokens, 1, -1, static_cast<const uint16_t*>(d_shared), H,
+                               static_cast<uint16_t*>(d_out), H, H, s);
+}

@@ -1,0 +1,59 @@
+// Internal launch interface of the decode kernels over the wave64 ("A64") packing, shared by
+// the single-expert entry points and the MoE layer driver.
+#pragma once
+
+#include "common.hpp"
+
+namespace aeon355 {
+
+// A segment is one expert with up to kSegTokens of its permuted positions: the unit of work of
+// the MFMA decode kernels (16 = the token dimension of v_mfma_f32_16x16x32_f16).
+constexpr int kSegTokens = 16;
+
+struct SegmentList {
+    const int* expert;  // [capacity] expert id of each segment
+    const int* first;   // [capacity] first permuted position
+    const int* count;   // [capacity] 1..kSegTokens
+    const int* total;   // [1] number of live segments (device); null = "direct" mode: one
+                        // segment, positions 0..direct_count-1 of direct_expert
+    int capacity;       // grid bound: blocks past *total exit at once
+};
+
+struct SegGateUpArgs {
+    const uint16_t* x;        // activations, fp16 bits
+    long x_stride;            // elements between token rows
+    const int* row_index;     // [positions] position -> activation row; null = identity
+    const aeon_a64_expert* experts;  // device table
+    SegmentList seg;
+    uint16_t* hidden;         // [positions][I] fp16
+    int H, I;
+    float limit;
+    aeon_a64_expert direct_expert;
+    int direct_count;
+};
+
+struct SegDownArgs {
+    const uint16_t* hidden;   // [positions][I] fp16
+    const aeon_a64_expert* experts;
+    SegmentList seg;
+    const int* out_row;       // [positions] position -> row of `contrib`; null = identity
+    const float* weight;      // [positions] routing weight of the position
+    float* contrib;           // [rows][H] fp32, one writer per element
+    int H, I;
+    aeon_a64_expert direct_expert;
+    int direct_count;
+};
+
+// k_split: 1, 2 or 4 waves of a workgroup share one 16-row tile and split K between them.
+int launch_seg_gate_up(const SegGateUpArgs& a, int k_split, hipStream_t stream);
+int launch_seg_down(const SegDownArgs& a, int k_split, hipStream_t stream);
+
+// out[t][i] = half( [shared: float(half(contrib[shared_base + t][i]))] +
+//                   sum_{s < slots, ascending} contrib[t*slots + s][i] ),
+// with `initial` (nullable, may alias out) added as the fp16 starting value when there is no
+// in-buffer shared row (shared_base < 0).
+int launch_token_reduce(const float* contrib, int tokens, int slots, int shared_base,
+                        const uint16_t* initial, long initial_stride, uint16_t* out,
+                        long out_stride, int hidden, hipStream_t stream);
+
+}  // namespace aeon355

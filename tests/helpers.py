@@ -1,0 +1,105 @@
+"""Helpers shared by the tests: synthetic experts in every layout, device upload, comparison."""
+import ctypes as C
+
+import numpy as np
+
+import orc
+from project_aeon_amd import capi, synth
+
+CFG13 = (4, 8)   # aeon::kCfgW13, aeon_w4a16_swizzle.hpp:14
+CFG2 = (8, 4)    # aeon::kCfgW2,  aeon_w4a16_swizzle.hpp:15
+
+
+def u32p(a):
+    return a.ctypes.data_as(C.POINTER(C.c_uint32))
+
+
+def u16p(a):
+    return a.ctypes.data_as(C.POINTER(C.c_uint16))
+
+
+class Matrix:
+    """One int4 matrix in the three layouts: source, `.aeon` swizzled (group-32 scales) and the
+    wave64 packing (group-128 scales, via the library's own host repack)."""
+
+    def __init__(self, packed_src, scale128, N, K, cfg):
+        self.N, self.K, self.cfg = N, K, cfg
+        self.src_packed = packed_src
+        self.scale128 = scale128
+        scale32 = np.ascontiguousarray(synth.scale32_from_scale128(scale128))
+        self.swz_packed, self.swz_scale = orc.swizzle(packed_src, scale32.view(np.uint16).ravel(),
+                                                      N, K, *cfg)
+        self.a64_packed = np.empty(N * K // 8, dtype=np.uint32)
+        self.a64_scale = np.empty(N * K // 128, dtype=np.uint16)
+        capi.call("aeon_a64_repack_host", u32p(self.swz_packed), u16p(self.swz_scale), N, K,
+                  cfg[0], cfg[1], u32p(self.a64_packed), u16p(self.a64_scale))
+
+    def decode(self):
+        return orc.swizzled_decode(self.swz_packed, self.swz_scale, self.N, self.K, *self.cfg)
+
+
+def synth_matrix(seed, expert, matrix, N, K):
+    cfg = CFG2 if matrix == synth.STREAM_W2 else CFG13
+    p, s = synth.expert_matrix_source(seed, expert, matrix, N, K)
+    return Matrix(p, s, N, K, cfg)
+
+
+class Expert:
+    def __init__(self, seed, expert, H, I):
+        self.H, self.I = H, I
+        self.w1 = synth_matrix(seed, expert, synth.STREAM_W1, I, H)
+        self.w3 = synth_matrix(seed, expert, synth.STREAM_W3, I, H)
+        self.w2 = synth_matrix(seed, expert, synth.STREAM_W2, H, I)
+
+    def ffn(self, x, limit, round_hidden=True, want_hidden=False):
+        """Oracle FFN of fp16 activations x [tokens][H] -> float64 [tokens][H]."""
+        return orc.expert_ffn((self.w1.swz_packed, self.w1.swz_scale),
+                              (self.w3.swz_packed, self.w3.swz_scale),
+                              (self.w2.swz_packed, self.w2.swz_scale), self.H, self.I,
+                              np.asarray(x, dtype=np.float64), limit, round_hidden=round_hidden,
+                              want_hidden=want_hidden)
+
+
+def to_dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def dev_u32(a):
+    """uint32 numpy -> device tensor (stored as int32 bits)."""
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int32)).cuda()
+
+
+def dev_u16(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).cuda()
+
+
+def dev_half(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float16)).cuda()
+
+
+class DevExpert:
+    """Device copies of an Expert in the wave64 packing plus the ctypes view of them."""
+
+    def __init__(self, e):
+        self.t = [dev_u32(e.w1.a64_packed), dev_u16(e.w1.a64_scale), dev_u32(e.w3.a64_packed),
+                  dev_u16(e.w3.a64_scale), dev_u32(e.w2.a64_packed), dev_u16(e.w2.a64_scale)]
+        self.c = capi.A64Expert(*[t.data_ptr() for t in self.t])
+
+
+def rel_err(got, want, floor_fraction=1e-3):
+    """max |got-want| / max(|want|, floor_fraction*max|want|): the relative error of
+    dsv4_oracle.hpp:96-129 (denominator floored at a fraction of the data's scale)."""
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    scale = np.abs(want).max()
+    denom = np.maximum(np.abs(want), floor_fraction * scale)
+    return float((np.abs(got - want) / denom).max())
+
+
+def stream_ptr():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)

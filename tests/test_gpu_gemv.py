@@ -1,0 +1,236 @@
+"""GPU parity: W4A16 GEMV / dual-GEMV (both layouts), the fused gate/up + SwiGLU, the W2
+contribution and the fixed-order reduce, against the fp64 oracle on the same seeded inputs.
+Tolerance: max relative error 1e-2 (denominator floored at 1e-3 of the peak), the bar for
+fp32-accumulate outputs; the reference's own GEMV gate allows 0.05 absolute
+(tests/test_w4a16_swizzled_gemv.cpp:122)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+def _setup():
+    import torch
+    assert torch.cuda.is_available()
+    import helpers
+    from project_aeon_amd import capi
+    return torch, helpers, capi
+
+
+def _reference_fixture(N, K):
+    """The closed-form fixture of tests/test_w4a16_swizzled_gemv.cpp:36-43,61-70, regenerated:
+    nibble j of word i = (3i + 5j + 1) % 16, scale i = 2^-8 * (1 + i % 29),
+    x[k] = ((k % 19) - 9) / 32."""
+    idx = np.arange(N * K // 8, dtype=np.uint64)
+    words = np.zeros(N * K // 8, dtype=np.uint32)
+    for j in range(8):
+        words |= (((idx * 3 + j * 5 + 1) % 16).astype(np.uint32)) << np.uint32(4 * j)
+    scale = (0.00390625 * (1 + np.arange(N * K // 32) % 29)).astype(np.float16)
+    x = (((np.arange(K) % 19) - 9) * 0.03125).astype(np.float16)
+    return words, scale, x
+
+
+@pytest.mark.parametrize("N,K,cfg", [(2048, 4096, (4, 8)), (4096, 2048, (8, 4))])
+def test_swizzled_gemv_reference_fixture(orc, N, K, cfg):
+    torch, h, capi = _setup()
+    words, scale, x = _reference_fixture(N, K)
+    swp, sws = orc.swizzle(words, scale.view(np.uint16), N, K, *cfg)
+    want = orc.swizzled_matvec(swp, sws, N, K, cfg[0], cfg[1], x.astype(np.float64))
+    d_x, d_p, d_s = h.dev_half(x), h.dev_u32(swp), h.dev_u16(sws)
+    out = torch.zeros(N, dtype=torch.float16, device="cuda")
+    capi.call("aeon_w4a16_swizzled_gemv", capi.vp(d_x), capi.vp(d_p), capi.vp(d_s), capi.vp(out),
+              N, K, cfg[0], cfg[1], h.stream_ptr())
+    got = out.cpu().numpy().astype(np.float64)
+    assert np.abs(got - want).max() < 0.05
+    assert h.rel_err(got, want) <= TOL
+    # a deliberately wrong reading (unsigned zero point) must be far away: the check is not vacuous
+    wrong = orc.swizzled_decode(swp, sws, N, K, cfg[0], cfg[1], signed_zp=False) @ x.astype(np.float64)
+    assert h.rel_err(wrong, want) > 10 * TOL
+
+
+def test_config0_single_gemv_both_layouts(orc):
+    """BASELINE config 0: x [1x7168] ~N(0,1), W int4 [7168->2048], group-128 scales, seed 0."""
+    torch, h, capi = _setup()
+    from project_aeon_amd import synth
+    N, K = 2048, 7168
+    m = h.synth_matrix(0, 0, synth.STREAM_W1, N, K)
+    x = synth.activations(0, 1, K)
+    want = orc.swizzled_matvec(m.swz_packed, m.swz_scale, N, K, 4, 8, x.astype(np.float64))[0]
+    d_x = h.dev_half(x)
+    out_swz = torch.zeros(N, dtype=torch.float16, device="cuda")
+    d_p, d_s = h.dev_u32(m.swz_packed), h.dev_u16(m.swz_scale)
+    capi.call("aeon_w4a16_swizzled_gemv", capi.vp(d_x), capi.vp(d_p), capi.vp(d_s),
+              capi.vp(out_swz), N, K, 4, 8, h.stream_ptr())
+    out_a64 = torch.zeros(N, dtype=torch.float16, device="cuda")
+    d_ap, d_as = h.dev_u32(m.a64_packed), h.dev_u16(m.a64_scale)
+    capi.call("aeon_a64_gemv", capi.vp(d_x), K, capi.vp(d_ap), capi.vp(d_as), capi.vp(out_a64), N,
+              1, N, K, h.stream_ptr())
+    for got in (out_swz, out_a64):
+        g = got.cpu().numpy().astype(np.float64)
+        assert np.abs(want).max() > 1.0
+        assert h.rel_err(g, want) <= TOL
+
+
+@pytest.mark.parametrize("tokens", [1, 2, 3, 8])
+@pytest.mark.parametrize("N,K,matrix", [(2048, 7168, 0), (7168, 2048, 2), (64, 256, 0)])
+def test_a64_gemv_and_dual(orc, tokens, N, K, matrix):
+    torch, h, capi = _setup()
+    from project_aeon_amd import synth
+    ma = h.synth_matrix(3, 1, matrix, N, K)
+    mb = h.synth_matrix(3, 2, matrix, N, K)
+    x = synth.activations(7, tokens, K)
+    want_a = orc.swizzled_matvec(ma.swz_packed, ma.swz_scale, N, K, *ma.cfg, x.astype(np.float64))
+    want_b = orc.swizzled_matvec(mb.swz_packed, mb.swz_scale, N, K, *mb.cfg, x.astype(np.float64))
+    d_x = h.dev_half(x)
+    pa, sa, pb, sb = (h.dev_u32(ma.a64_packed), h.dev_u16(ma.a64_scale), h.dev_u32(mb.a64_packed),
+                      h.dev_u16(mb.a64_scale))
+    single = torch.zeros(tokens, N, dtype=torch.float16, device="cuda")
+    capi.call("aeon_a64_gemv", capi.vp(d_x), K, capi.vp(pa), capi.vp(sa), capi.vp(single), N,
+              tokens, N, K, h.stream_ptr())
+    oa = torch.zeros(tokens, N, dtype=torch.float16, device="cuda")
+    ob = torch.zeros(tokens, N, dtype=torch.float16, device="cuda")
+    capi.call("aeon_a64_dual_gemv", capi.vp(d_x), K, capi.vp(pa), capi.vp(sa), capi.vp(pb),
+              capi.vp(sb), capi.vp(oa), capi.vp(ob), N, tokens, N, K, h.stream_ptr())
+    assert h.rel_err(single.cpu().numpy(), want_a) <= TOL
+    assert h.rel_err(oa.cpu().numpy(), want_a) <= TOL
+    assert h.rel_err(ob.cpu().numpy(), want_b) <= TOL
+    # the dual kernel is two single launches sharing one activation read: bit-equal
+    # (tests/test_w4a16_swizzled_dual_gemv.cpp)
+    assert torch.equal(single, oa)
+
+
+def test_swizzled_dual_equals_two_singles(orc):
+    torch, h, capi = _setup()
+    from project_aeon_amd import synth
+    N, K = 2048, 4096
+    ma = h.synth_matrix(1, 0, 0, N, K)
+    mb = h.synth_matrix(7, 0, 1, N, K)
+    x = synth.activations(1, 1, K)
+    d_x = h.dev_half(x)
+    pa, sa, pb, sb = (h.dev_u32(ma.swz_packed), h.dev_u16(ma.swz_scale), h.dev_u32(mb.swz_packed),
+                      h.dev_u16(mb.swz_scale))
+    outs = [torch.zeros(N, dtype=torch.float16, device="cuda") for _ in range(4)]
+    capi.call("aeon_w4a16_swizzled_gemv", capi.vp(d_x), capi.vp(pa), capi.vp(sa), capi.vp(outs[0]),
+              N, K, 4, 8, h.stream_ptr())
+    capi.call("aeon_w4a16_swizzled_gemv", capi.vp(d_x), capi.vp(pb), capi.vp(sb), capi.vp(outs[1]),
+              N, K, 4, 8, h.stream_ptr())
+    capi.call("aeon_w4a16_swizzled_dual_gemv", capi.vp(d_x), capi.vp(pa), capi.vp(sa), capi.vp(pb),
+              capi.vp(sb), capi.vp(outs[2]), capi.vp(outs[3]), N, K, 4, 8, h.stream_ptr())
+    assert torch.equal(outs[0], outs[2]) and torch.equal(outs[1], outs[3])
+    want = orc.swizzled_matvec(ma.swz_packed, ma.swz_scale, N, K, 4, 8, x.astype(np.float64))[0]
+    assert h.rel_err(outs[2].cpu().numpy(), want) <= TOL
+
+
+def test_gemv_rejects_bad_shapes():
+    torch, h, capi = _setup()
+    t = torch.zeros(4096, dtype=torch.float16, device="cuda")
+    with pytest.raises(ValueError):  # K != iters*lpr*32
+        capi.call("aeon_w4a16_swizzled_gemv", capi.vp(t), capi.vp(t), capi.vp(t), capi.vp(t), 64,
+                  100, 4, 8, None)
+    with pytest.raises(ValueError):  # N % rpw
+        capi.call("aeon_w4a16_swizzled_gemv", capi.vp(t), capi.vp(t), capi.vp(t), capi.vp(t), 6,
+                  256, 4, 8, None)
+    with pytest.raises(ValueError):  # null
+        capi.call("aeon_w4a16_swizzled_gemv", None, capi.vp(t), capi.vp(t), capi.vp(t), 64, 256,
+                  4, 8, None)
+    with pytest.raises(ValueError):
+        capi.call("aeon_a64_gemv", capi.vp(t), 256, capi.vp(t), capi.vp(t), capi.vp(t), 64, 9, 64,
+                  256, None)
+
+
+@pytest.mark.parametrize("experts", [1, 6, 8])
+def test_swizzled_expert_trio_reference_shapes(orc, experts):
+    """The per-token trio of v4_expert_executor.hpp:340-369 on the reference's own shapes
+    (hidden 4096, intermediate 2048, group 32) and the payload family of
+    tests/test_moe_grouped_batch_parity.cpp:73-91 (byte pattern, power-of-two scales)."""
+    torch, h, capi = _setup()
+    H, I, limit = 4096, 2048, 10.0
+    rng = np.random.default_rng(0xC0FFEE)
+    x = (rng.random(H) - 0.5).astype(np.float16)
+    weights = (0.6 / (np.arange(experts) + 1) + 0.02).astype(np.float32)
+    w13, w2 = capi.W13Table(), capi.W2Table()
+    keep, mats = [], []
+    for e in range(experts):
+        def payload(n_words, seed):
+            i = np.arange(n_words * 4, dtype=np.uint64)
+            return ((i * 37 + seed * 11) & 0xFF).astype(np.uint8).view(np.uint32)
+        def scales(n):
+            return np.ldexp(1.0, -6 + (np.arange(n) % 4)).astype(np.float16).view(np.uint16)
+        m = {}
+        for name, rows, cols in (("w1", I, H), ("w3", I, H), ("w2", H, I)):
+            m[name] = (payload(rows * cols // 8, e * 3 + len(m)), scales(rows * cols // 32))
+        mats.append(m)
+        dev = {k: (h.dev_u32(v[0]), h.dev_u16(v[1])) for k, v in m.items()}
+        keep.append(dev)
+        w13.w1[e], w13.s1[e] = dev["w1"][0].data_ptr(), dev["w1"][1].data_ptr()
+        w13.w3[e], w13.s3[e] = dev["w3"][0].data_ptr(), dev["w3"][1].data_ptr()
+        w2.w2[e], w2.s2[e] = dev["w2"][0].data_ptr(), dev["w2"][1].data_ptr()
+    d_x = h.dev_half(x)
+    hidden = torch.zeros(8, I, dtype=torch.float16, device="cuda")
+    contrib = torch.zeros(experts, H, dtype=torch.float32, device="cuda")
+    shared = h.dev_half((rng.random(H) - 0.5).astype(np.float16))
+    out = shared.clone()
+    d_w = h.to_dev(weights)
+    capi.call("aeon_moe_gemv_w13_swiglu", capi.vp(d_x), C.byref(w13), capi.vp(hidden), None, I,
+              experts, I, H, 4, 8, C.c_float(limit), h.stream_ptr())
+    capi.call("aeon_moe_fused_w2_contrib", capi.vp(hidden), C.byref(w2), capi.vp(d_w),
+              capi.vp(contrib), experts, H, I, 8, 4, h.stream_ptr())
+    capi.call("aeon_moe_accumulate_fixed_order", capi.vp(contrib), experts, capi.vp(out),
+              capi.vp(out), H, h.stream_ptr())
+    got_hidden = hidden.cpu().numpy()[:experts].astype(np.float64)
+    got_contrib = contrib.cpu().numpy().astype(np.float64)
+    want_contrib = np.empty((experts, H))
+    for e, m in enumerate(mats):
+        o, hid = orc.expert_ffn(m["w1"], m["w3"], m["w2"], H, I, x.astype(np.float64), limit,
+                                round_hidden=True, want_hidden=True)
+        assert h.rel_err(got_hidden[e], hid) <= TOL
+        want_contrib[e] = float(weights[e]) * o
+    assert h.rel_err(got_contrib, want_contrib) <= TOL
+    # contrib == weight x unit-weight contribution, bit for bit (tests/test_v4_moe_accum_oracle.cpp)
+    unit = torch.zeros_like(contrib)
+    capi.call("aeon_moe_fused_w2_contrib", capi.vp(hidden), C.byref(w2),
+              capi.vp(torch.ones(experts, device="cuda")), capi.vp(unit), experts, H, I, 8, 4,
+              h.stream_ptr())
+    assert torch.equal(contrib, unit * d_w[:, None])
+    # fixed-order reduce: fp32 slot-order sum with the shared value as the initial term, one rounding
+    acc = shared.float()
+    for e in range(experts):
+        acc = acc + contrib[e]
+    assert torch.equal(out, acc.half())
+    want_out = orc.moe_combine(want_contrib, shared.cpu().numpy().astype(np.float64))
+    assert h.rel_err(out.cpu().numpy(), want_out) <= TOL
+
+
+@pytest.mark.parametrize("use_mfma", [0, 1])
+@pytest.mark.parametrize("tokens", [1, 4, 8])
+def test_config1_one_expert_decode(orc, tokens, use_mfma):
+    """BASELINE config 1: one routed expert, batch 1/4/8, H=7168, I=2048, clamp 7, output scaled
+    by a router weight in (0,1]."""
+    torch, h, capi = _setup()
+    from project_aeon_amd import synth
+    H, I, limit = 7168, 2048, 7.0
+    e = h.Expert(0, 0, H, I)
+    de = h.DevExpert(e)
+    x = synth.activations(0, tokens, H)
+    w = synth.route_weights(0, tokens)
+    d_x, d_w = h.dev_half(x), h.to_dev(w)
+    hidden = torch.zeros(tokens, I, dtype=torch.float16, device="cuda")
+    contrib = torch.zeros(tokens, H, dtype=torch.float32, device="cuda")
+    out = torch.zeros(tokens, H, dtype=torch.float16, device="cuda")
+    capi.call("aeon_a64_expert_decode", capi.vp(d_x), tokens, C.byref(de.c), capi.vp(d_w),
+              capi.vp(hidden), capi.vp(contrib), None, capi.vp(out), H, I, C.c_float(limit),
+              use_mfma, h.stream_ptr())
+    want, want_hidden = e.ffn(x, limit, round_hidden=True, want_hidden=True)
+    want = want * w.astype(np.float64)[:, None]
+    assert np.abs(want).max() > 1.0
+    assert h.rel_err(hidden.cpu().numpy(), want_hidden) <= TOL
+    assert h.rel_err(contrib.cpu().numpy(), want) <= TOL
+    assert h.rel_err(out.cpu().numpy(), want) <= TOL
+    assert torch.equal(out, contrib.half())
+    # the unrounded-hidden oracle (dsv4_oracle.hpp:1633-1671 keeps hidden in fp64) agrees too
+    assert h.rel_err(out.cpu().numpy(), e.ffn(x, limit, round_hidden=False) *
+                     w.astype(np.float64)[:, None]) <= TOL

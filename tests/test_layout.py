@@ -1,0 +1,91 @@
+"""The weight layouts on the host: the library's swizzle against the oracle's, and the wave64
+repack checked bit-exact (round trip, address closed form, dequantised values)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from helpers import CFG13, CFG2, Matrix, synth_matrix, u16p, u32p
+from project_aeon_amd import capi, synth
+
+
+@pytest.mark.parametrize("N,K,cfg", [(2048, 7168, CFG13), (7168, 2048, CFG2), (16, 256, CFG13),
+                                     (32, 128, CFG2), (2048, 4096, CFG13), (4096, 2048, CFG2)])
+def test_swizzle_matches_oracle_and_roundtrips(orc, N, K, cfg):
+    rng = np.random.default_rng(N + K)
+    sp = rng.integers(0, 2**32, N * K // 8, dtype=np.uint32)
+    ss = rng.integers(0, 2**16, N * K // 32, dtype=np.uint16)
+    dp, ds = np.empty_like(sp), np.empty_like(ss)
+    capi.call("aeon_swizzle_w4a16", u32p(sp), u16p(ss), u32p(dp), u16p(ds), N, K, *cfg)
+    op, os_ = orc.swizzle(sp, ss, N, K, *cfg)
+    assert np.array_equal(dp, op) and np.array_equal(ds, os_)
+    bp, bs = np.empty_like(sp), np.empty_like(ss)
+    capi.call("aeon_unswizzle_w4a16", u32p(dp), u16p(ds), u32p(bp), u16p(bs), N, K, *cfg)
+    assert np.array_equal(bp, sp) and np.array_equal(bs, ss)
+
+
+def test_swizzle_rejects_bad_shapes():
+    a = np.zeros(64, dtype=np.uint32)
+    s = np.zeros(64, dtype=np.uint16)
+    for N, K, rpw, lpr in [(6, 256, 4, 8), (8, 100, 4, 8), (8, 256, 4, 4), (8, 128, 4, 8), (0, 256, 4, 8)]:
+        with pytest.raises(ValueError):
+            capi.call("aeon_swizzle_w4a16", u32p(a), u16p(s), u32p(a), u16p(s), N, K, rpw, lpr)
+
+
+@pytest.mark.parametrize("N,K,matrix", [(2048, 7168, synth.STREAM_W1), (7168, 2048, synth.STREAM_W2),
+                                        (16, 256, synth.STREAM_W1), (48, 384, synth.STREAM_W2)])
+def test_a64_repack_bit_exact(orc, N, K, matrix):
+    m = synth_matrix(0, 5, matrix, N, K)
+    # the oracle packs straight from the source layout; the library repacks the swizzled payload
+    op, os_ = orc.a64_pack(m.src_packed, synth.scale32_from_scale128(m.scale128).view(np.uint16),
+                           N, K)
+    assert np.array_equal(m.a64_packed, op)
+    assert np.array_equal(m.a64_scale, os_)
+    # round trip back to the `.aeon` payload
+    bp, bs = np.empty_like(m.swz_packed), np.empty_like(m.swz_scale)
+    capi.call("aeon_a64_unrepack_host", u32p(m.a64_packed), u16p(m.a64_scale), N, K, m.cfg[0],
+              m.cfg[1], u32p(bp), u16p(bs))
+    assert np.array_equal(bp, m.swz_packed) and np.array_equal(bs, m.swz_scale)
+    assert capi.lib().aeon_a64_packed_bytes(N, K) == m.a64_packed.nbytes
+    assert capi.lib().aeon_a64_scale_bytes(N, K) == m.a64_scale.nbytes
+
+
+def test_a64_dequantised_weights_bit_exact(orc):
+    # every element of a small matrix, through both layouts' decoders
+    m = synth_matrix(1, 2, synth.STREAM_W1, 64, 512)
+    want = m.decode()
+    got = orc.a64_decode(m.a64_packed, m.a64_scale, 64, 512)
+    assert np.array_equal(got, want)
+    # and through the source layout by hand: (q-8)*scale with q at nibble k%8
+    q = (m.src_packed.reshape(64, 64)[:, :, None] >> (4 * np.arange(8, dtype=np.uint32))) & 0xF
+    w = (q.reshape(64, 512).astype(np.float64) - 8.0) * np.repeat(m.scale128.astype(np.float64), 128, axis=1)
+    assert np.array_equal(w, want)
+    assert np.array_equal(np.float32(w).astype(np.float64), w)  # exact in fp32 as well
+
+
+def test_a64_full_size_checksum(orc):
+    # full-size matrix: sampled elements + a checksum of checksums instead of 14.7M decodes
+    N, K = 2048, 7168
+    m = synth_matrix(0, 0, synth.STREAM_W1, N, K)
+    rng = np.random.default_rng(0)
+    for _ in range(4000):
+        r, c = int(rng.integers(N)), int(rng.integers(K))
+        pw, nib, si = orc.a64_address(K, r, c)
+        q = (int(m.a64_packed[pw]) >> (4 * nib)) & 0xF
+        qs = (int(m.src_packed[r * (K // 8) + c // 8]) >> (4 * (c % 8))) & 0xF
+        assert q == qs and m.a64_scale[si] == m.scale128.view(np.uint16)[r, c // 128]
+    assert int(m.a64_packed.astype(np.uint64).sum()) == int(m.swz_packed.astype(np.uint64).sum())
+
+
+def test_a64_repack_rejects_unequal_group32_scales(orc):
+    N, K = 16, 256
+    p, s128 = synth.expert_matrix_source(0, 0, synth.STREAM_W1, N, K)
+    s32 = np.ascontiguousarray(synth.scale32_from_scale128(s128)).view(np.uint16)
+    s32[3, 5] ^= 1
+    swp, sws = orc.swizzle(p, s32.ravel(), N, K, *CFG13)
+    out_p = np.empty(N * K // 8, dtype=np.uint32)
+    out_s = np.empty(N * K // 128, dtype=np.uint16)
+    with pytest.raises(ValueError, match="group-32"):
+        capi.call("aeon_a64_repack_host", u32p(swp), u16p(sws), N, K, 4, 8, u32p(out_p), u16p(out_s))
+    with pytest.raises(ValueError):
+        capi.call("aeon_a64_repack_host", u32p(swp), u16p(sws), 8, 256, 4, 8, u32p(out_p), u16p(out_s))
