@@ -59,6 +59,11 @@ class Expert:
                               np.asarray(x, dtype=np.float64), limit, round_hidden=round_hidden,
                               want_hidden=want_hidden)
 
+    def down(self, hidden):
+        """Oracle W2 over given hidden rows [tokens][I] -> float64 [tokens][H]."""
+        return orc.swizzled_matvec(self.w2.swz_packed, self.w2.swz_scale, self.H, self.I,
+                                   *self.w2.cfg, np.asarray(hidden, dtype=np.float64))
+
 
 def to_dev(a):
     import torch

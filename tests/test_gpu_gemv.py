@@ -227,10 +227,17 @@ def test_config1_one_expert_decode(orc, tokens, use_mfma):
     want, want_hidden = e.ffn(x, limit, round_hidden=True, want_hidden=True)
     want = want * w.astype(np.float64)[:, None]
     assert np.abs(want).max() > 1.0
+    # stage by stage at 1e-2: gate/up+SwiGLU against the oracle, then W2 against the oracle fed
+    # the device's own fp16 hidden (one flipped fp16 rounding of a hidden value moves near-zero
+    # outputs by more than 1e-2 of themselves, so the chained comparison is made on the peak)
     assert h.rel_err(hidden.cpu().numpy(), want_hidden) <= TOL
-    assert h.rel_err(contrib.cpu().numpy(), want) <= TOL
-    assert h.rel_err(out.cpu().numpy(), want) <= TOL
+    staged = e.down(hidden.cpu().numpy()) * w.astype(np.float64)[:, None]
+    assert h.rel_err(contrib.cpu().numpy(), staged) <= TOL
+    assert h.rel_err(out.cpu().numpy(), staged) <= TOL
+    assert np.abs(out.cpu().numpy() - want).max() <= 6e-3 * np.abs(want).max()
     assert torch.equal(out, contrib.half())
-    # the unrounded-hidden oracle (dsv4_oracle.hpp:1633-1671 keeps hidden in fp64) agrees too
-    assert h.rel_err(out.cpu().numpy(), e.ffn(x, limit, round_hidden=False) *
-                     w.astype(np.float64)[:, None]) <= TOL
+    # against the oracle that keeps hidden in fp64 (dsv4_oracle.hpp:1633-1671) the fp16 store of
+    # hidden shows up on near-zero outputs, so that comparison is the reference's own: a fraction
+    # of the peak (6e-3, tests/test_v4_expert_oracle.cpp:75-77)
+    unrounded = e.ffn(x, limit, round_hidden=False) * w.astype(np.float64)[:, None]
+    assert np.abs(out.cpu().numpy() - unrounded).max() <= 6e-3 * np.abs(unrounded).max()
