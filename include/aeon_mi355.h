@@ -164,6 +164,97 @@ int aeon_a64_expert_decode(const void* d_x, int tokens, const aeon_a64_expert* e
                            const void* d_shared, void* d_out, int H, int I, float swiglu_limit,
                            int use_mfma, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Router, permutation, and one MoE layer on the device
+ * ---------------------------------------------------------------------------------------- */
+
+#define AEON_ROUTER_SCORE_SQRT_SOFTPLUS 0 /* sqrt(softplus(x)), moe_router.hpp:17-27 */
+#define AEON_ROUTER_SCORE_SIGMOID 1       /* 1/(1+exp(-x)) */
+
+/* Router logits: logits[t][e] = sum_h float(x[t][h]) * Wr[h][e], Wr fp32 [hidden][experts].
+ * Replaces the gate GEMV + widening of dispatch_router (src/architecture/deepseek_v4/layer/
+ * v4_layer_body_moe.hpp:124-159, gemv_fp16_vec8_kernel in src/platform/ops/gemv.hpp:72-110)
+ * for an fp32 gate. Accumulation order is fixed (h ascending inside a chunk, chunks ascending),
+ * so a run is bit-reproducible. The workspace holds the per-chunk partial sums. */
+size_t aeon_router_logits_workspace_bytes(int tokens, int hidden, int experts);
+int aeon_router_logits(const void* d_x, int x_stride, const float* d_router_weight,
+                       float* d_logits, int tokens, int hidden, int experts, void* d_workspace,
+                       size_t workspace_bytes, void* stream);
+
+/* moe_router_kernel launch (src/architecture/deepseek_v4/kernels/moe_router.hpp:104-189; host
+ * twin cpu_moe_router :29-100): score = f(logit); choice = score + bias (bias added after the
+ * activation, nullable); ids = top_k by descending choice, ties to the lowest index; weights =
+ * unbiased score / (sum + 1e-20) [if renormalize] * routed_scaling_factor. With a hash table
+ * ([vocab][top_k] int64) and token ids the ids come from the table instead (:146-153).
+ * experts <= 1024, top_k <= 64. Scores and selection are evaluated in fp64. */
+int aeon_moe_router(const float* d_logits, const float* d_bias, const int64_t* d_hash_table,
+                    const int32_t* d_token_ids, float* d_topk_weights, int32_t* d_topk_indices,
+                    int tokens, int experts, int top_k, float routed_scaling_factor,
+                    int renormalize, int score_kind, void* stream);
+
+/* dispatch_expert_permutation, src/platform/ops/expert_permutation.hpp:130-175: ids
+ * [token_count*slots] -> expert_offsets [expert_count+1], token_indices and draw_indices
+ * [token_count*slots] (ascending draw inside an expert), and optionally the weights gathered
+ * into position order. expert_count <= 1024; ids outside [0, expert_count) are dropped. */
+int aeon_expert_permutation(const int32_t* d_topk_indices, int token_count, int slots,
+                            int expert_count, int32_t* d_expert_offsets, int32_t* d_token_indices,
+                            int32_t* d_draw_indices, const float* d_weights_by_draw,
+                            float* d_weights_by_position, void* stream);
+
+/* One MoE layer with every expert resident in HBM in the wave64 packing. `d_experts` is a
+ * DEVICE array of `experts` entries (+1 when has_shared: the last entry is the always-on
+ * expert) -- a table in memory instead of the 8-entry by-value tables of
+ * aeon_moe_fused_w13.hpp:13-20, so one launch can address every expert of the layer. */
+typedef struct {
+    int hidden;
+    int intermediate;
+    int experts;  /* routed experts */
+    int top_k;
+    int has_shared;
+    float swiglu_limit;
+    int score_kind;
+    float routed_scaling_factor;
+    int renormalize;
+    const float* d_router_weight; /* fp32 [hidden][experts]; only aeon_moe_layer_decode reads it */
+    const float* d_router_bias;   /* fp32 [experts], nullable */
+    const aeon_a64_expert* d_experts;
+} aeon_moe_layer;
+
+size_t aeon_moe_layer_workspace_bytes(const aeon_moe_layer* layer, int max_tokens);
+
+/* V4RoutedExpertExecutor::accumulate_routed_batch for resident experts
+ * (src/architecture/deepseek_v4/layer/v4_layer_body_moe.hpp:76-105, production override
+ * src/architecture/deepseek_v4/moe/v4_expert_executor.hpp:379-461) at decode batch sizes:
+ * given the routed ids/weights [tokens][top_k] on the device, out[t] = half(shared(x_t) as fp16
+ * + sum_k w[t][k] * expert_{ids[t][k]}(x_t)) in slot order, fp32. Without a shared expert the
+ * value already in d_out is the fp16 starting value, as moe_accum is in the reference. Each
+ * distinct expert's weights are streamed once per 16 of its tokens. No host synchronisation. */
+int aeon_moe_layer_routed(const aeon_moe_layer* layer, const void* d_x, int x_stride, int tokens,
+                          const int32_t* d_topk_ids, const float* d_topk_weights, void* d_out,
+                          int out_stride, void* d_workspace, size_t workspace_bytes, void* stream);
+
+/* Router + aeon_moe_layer_routed: the device half of run_layer_body_router
+ * (v4_layer_body_moe.hpp:168-202) followed by run_layer_body_moe_and_post's expert part
+ * (:285-312), with the per-layer D2H read-back and stream synchronisation of :188-192 removed.
+ * d_topk_ids / d_topk_weights [tokens][top_k] are outputs. */
+int aeon_moe_layer_decode(const aeon_moe_layer* layer, const void* d_x, int x_stride, int tokens,
+                          void* d_out, int out_stride, int32_t* d_topk_ids, float* d_topk_weights,
+                          void* d_workspace, size_t workspace_bytes, void* stream);
+/* Device pointer to the fp32 logits [tokens][experts] the last aeon_moe_layer_decode call with
+ * this workspace and token count left behind (what the ids were selected from). */
+const float* aeon_moe_layer_logits(const aeon_moe_layer* layer, int tokens, void* d_workspace);
+
+/* ------------------------------------------------------------------------------------------
+ * Synthetic experts on the device (benchmarks and tests)
+ * ---------------------------------------------------------------------------------------- */
+
+/* Fills one matrix (matrix 0 = W1, 1 = W3, 2 = W2) of synthetic expert `expert` directly in
+ * device memory in the `.aeon` swizzled layout (packed N*K/2 bytes, scales N*K/32 fp16 with
+ * each group-128 scale replicated over its four group-32 slots): int4 uniform in [-8,7],
+ * scales uniform in [0.005,0.02], a pure function of (seed, expert, matrix, index). */
+int aeon_synth_matrix_swizzled(uint64_t seed, int expert, int matrix, int N, int K, int rpw,
+                               int lpr, void* d_packed, void* d_scale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -54,9 +54,8 @@ def lib():
         _lib.aeon_last_error.restype = C.c_char_p
         _lib.aeon_a64_packed_bytes.restype = C.c_size_t
         _lib.aeon_a64_scale_bytes.restype = C.c_size_t
-        for name in ("aeon_moe_layer_workspace_bytes",):
-            if hasattr(_lib, name):
-                getattr(_lib, name).restype = C.c_size_t
+        _lib.aeon_moe_layer_workspace_bytes.restype = C.c_size_t
+        _lib.aeon_router_logits_workspace_bytes.restype = C.c_size_t
     return _lib
 
 

@@ -1,0 +1,201 @@
+// One MoE layer over a batch of tokens, entirely on the caller's stream with no host
+// synchronisation: router logits -> top-k -> permutation + segments -> gate/up + SwiGLU ->
+// W2 x routing weight -> fixed-order reduce with the always-on expert as the initial value.
+// Routed ids, permutation and segment bounds stay in device memory; launch grids are sized by
+// their upper bounds and workgroups past the live count exit at once.
+#include "expert_a64.hpp"
+#include "permutation.hpp"
+
+extern "C" size_t aeon_router_logits_workspace_bytes(int tokens, int hidden, int experts);
+
+namespace aeon355 {
+
+static size_t align_up(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
+
+struct LayerWorkspace {
+    float* logits_partial;
+    float* logits;
+    int32_t* offsets;
+    int32_t* token_indices;
+    int32_t* draw_indices;
+    float* weights_by_position;
+    int32_t* seg_expert;
+    int32_t* seg_first;
+    int32_t* seg_count;
+    int32_t* seg_total;
+    uint16_t* hidden;
+    float* contrib;
+    int positions;
+    int seg_capacity;
+    size_t bytes;
+};
+
+static LayerWorkspace carve(const aeon_moe_layer& L, int tokens, void* base) {
+    LayerWorkspace w{};
+    const int draws = tokens * L.top_k;
+    w.positions = draws + (L.has_shared ? tokens : 0);
+    const int lists = L.experts + (L.has_shared ? 1 : 0);
+    // every list can end in one short segment; full segments are bounded by the positions
+    w.seg_capacity = lists + w.positions / kSegTokens + 1;
+    size_t at = 0;
+    char* p = static_cast<char*>(base);
+    auto take = [&](size_t bytes) {
+        char* here = p != nullptr ? p + at : nullptr;
+        at += align_up(bytes);
+        return here;
+    };
+    w.logits_partial = reinterpret_cast<float*>(
+        take(aeon_router_logits_workspace_bytes(tokens, L.hidden, L.experts)));
+    w.logits = reinterpret_cast<float*>(take(sizeof(float) * tokens * L.experts));
+    w.offsets = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * (lists + 1)));
+    w.token_indices = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * w.positions));
+    w.draw_indices = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * w.positions));
+    w.weights_by_position = reinterpret_cast<float*>(take(sizeof(float) * w.positions));
+    w.seg_expert = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * w.seg_capacity));
+    w.seg_first = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * w.seg_capacity));
+    w.seg_count = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * w.seg_capacity));
+    w.seg_total = reinterpret_cast<int32_t*>(take(sizeof(int32_t)));
+    w.hidden = reinterpret_cast<uint16_t*>(take(sizeof(uint16_t) * w.positions * L.intermediate));
+    w.contrib = reinterpret_cast<float*>(take(sizeof(float) * static_cast<size_t>(w.positions) * L.hidden));
+    w.bytes = at;
+    return w;
+}
+
+static int check_layer(const aeon_moe_layer* L, const char* who) {
+    AEON_REQUIRE(L != nullptr, AEON_ERR_INVALID_ARGUMENT, "%s: null layer", who);
+    AEON_REQUIRE(L->hidden > 0 && L->intermediate > 0 && L->hidden % 128 == 0 &&
+                     L->intermediate % 128 == 0,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: hidden and intermediate must be multiples of 128 "
+                 "(hidden=%d intermediate=%d)", who, L->hidden, L->intermediate);
+    AEON_REQUIRE(L->experts > 0 && L->experts + (L->has_shared ? 1 : 0) <= kMaxPermutationExperts &&
+                     L->top_k > 0 && L->top_k <= L->experts && L->top_k <= 64,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: bad expert geometry (experts=%d top_k=%d)", who,
+                 L->experts, L->top_k);
+    AEON_REQUIRE(L->d_experts != nullptr, AEON_ERR_INVALID_ARGUMENT, "%s: null expert table", who);
+    return AEON_OK;
+}
+
+}  // namespace aeon355
+
+using namespace aeon355;
+
+extern "C" int aeon_router_logits(const void*, int, const float*, float*, int, int, int, void*,
+                                  size_t, void*);
+extern "C" int aeon_moe_router(const float*, const float*, const int64_t*, const int32_t*, float*,
+                               int32_t*, int, int, int, float, int, int, void*);
+
+extern "C" size_t aeon_moe_layer_workspace_bytes(const aeon_moe_layer* layer, int max_tokens) {
+    if (layer == nullptr || max_tokens <= 0) return 0;
+    return carve(*layer, max_tokens, nullptr).bytes;
+}
+
+extern "C" int aeon_moe_layer_routed(const aeon_moe_layer* layer, const void* d_x, int x_stride,
+                                     int tokens, const int32_t* d_topk_ids,
+                                     const float* d_topk_weights, void* d_out, int out_stride,
+                                     void* d_workspace, size_t workspace_bytes, void* stream) {
+    const char* who = "aeon_moe_layer_routed";
+    if (int rc = check_layer(layer, who)) return rc;
+    AEON_REQUIRE(d_x && d_topk_ids && d_topk_weights && d_out && d_workspace,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
+    AEON_REQUIRE(tokens >= 0 && x_stride >= layer->hidden && x_stride % 8 == 0 &&
+                     out_stride >= layer->hidden,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: bad token shape (tokens=%d x_stride=%d out_stride=%d)",
+                 who, tokens, x_stride, out_stride);
+    if (tokens == 0) return AEON_OK;
+    const LayerWorkspace w = carve(*layer, tokens, d_workspace);
+    AEON_REQUIRE(workspace_bytes >= w.bytes, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: workspace of %zu bytes, %zu needed", who, workspace_bytes, w.bytes);
+    hipStream_t s = as_stream(stream);
+    const int draws = tokens * layer->top_k;
+
+    PermutationArgs p{};
+    p.ids = d_topk_ids;
+    p.draws = draws;
+    p.slots = layer->top_k;
+    p.experts = layer->experts;
+    p.shared_tokens = layer->has_shared ? tokens : 0;
+    p.offsets = w.offsets;
+    p.token_indices = w.token_indices;
+    p.draw_indices = w.draw_indices;
+    p.weights_by_draw = d_topk_weights;
+    p.weights_by_position = w.weights_by_position;
+    p.seg_expert = w.seg_expert;
+    p.seg_first = w.seg_first;
+    p.seg_count = w.seg_count;
+    p.seg_total = w.seg_total;
+    p.seg_tokens = kSegTokens;
+    p.seg_capacity = w.seg_capacity;
+    if (int rc = launch_permutation(p, s)) return rc;
+
+    // Few live segments (a small batch) leave the chip idle unless K is also split.
+    const int live_bound = (layer->has_shared ? (tokens + kSegTokens - 1) / kSegTokens : 0) +
+                           (draws < layer->experts ? draws : layer->experts);
+    const int split_gate = live_bound * (layer->intermediate / 16) >= 8192 ? 1 : 4;
+    const int split_down = live_bound * (layer->hidden / 16) >= 8192 ? 1 : 4;
+
+    SegGateUpArgs gu{};
+    gu.x = static_cast<const uint16_t*>(d_x);
+    gu.x_stride = x_stride;
+    gu.row_index = w.token_indices;
+    gu.experts = layer->d_experts;
+    gu.seg = SegmentList{w.seg_expert, w.seg_first, w.seg_count, w.seg_total, w.seg_capacity};
+    gu.hidden = w.hidden;
+    gu.H = layer->hidden;
+    gu.I = layer->intermediate;
+    gu.limit = layer->swiglu_limit;
+    if (int rc = launch_seg_gate_up(gu, split_gate, s)) return rc;
+
+    SegDownArgs dn{};
+    dn.hidden = w.hidden;
+    dn.experts = layer->d_experts;
+    dn.seg = gu.seg;
+    dn.out_row = w.draw_indices;
+    dn.weight = w.weights_by_position;
+    dn.contrib = w.contrib;
+    dn.H = layer->hidden;
+    dn.I = layer->intermediate;
+    if (int rc = launch_seg_down(dn, split_down, s)) return rc;
+
+    return launch_token_reduce(w.contrib, tokens, layer->top_k, layer->has_shared ? draws : -1,
+                               layer->has_shared ? nullptr : static_cast<const uint16_t*>(d_out),
+                               out_stride, static_cast<uint16_t*>(d_out), out_stride, layer->hidden, s);
+}
+
+extern "C" int aeon_moe_layer_decode(const aeon_moe_layer* layer, const void* d_x, int x_stride,
+                                     int tokens, void* d_out, int out_stride, int32_t* d_topk_ids,
+                                     float* d_topk_weights, void* d_workspace,
+                                     size_t workspace_bytes, void* stream) {
+    const char* who = "aeon_moe_layer_decode";
+    if (int rc = check_layer(layer, who)) return rc;
+    AEON_REQUIRE(layer->d_router_weight != nullptr, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: the layer has no router weight", who);
+    AEON_REQUIRE(d_x && d_out && d_topk_ids && d_topk_weights && d_workspace,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
+    AEON_REQUIRE(tokens >= 0 && x_stride >= layer->hidden, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: bad token shape (tokens=%d x_stride=%d)", who, tokens, x_stride);
+    if (tokens == 0) return AEON_OK;
+    const LayerWorkspace w = carve(*layer, tokens, d_workspace);
+    AEON_REQUIRE(workspace_bytes >= w.bytes, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: workspace of %zu bytes, %zu needed", who, workspace_bytes, w.bytes);
+    if (int rc = aeon_router_logits(d_x, x_stride, layer->d_router_weight, w.logits, tokens,
+                                    layer->hidden, layer->experts, w.logits_partial,
+                                    aeon_router_logits_workspace_bytes(tokens, layer->hidden,
+                                                                       layer->experts),
+                                    stream)) {
+        return rc;
+    }
+    if (int rc = aeon_moe_router(w.logits, layer->d_router_bias, nullptr, nullptr, d_topk_weights,
+                                 d_topk_ids, tokens, layer->experts, layer->top_k,
+                                 layer->routed_scaling_factor, layer->renormalize,
+                                 layer->score_kind, stream)) {
+        return rc;
+    }
+    return aeon_moe_layer_routed(layer, d_x, x_stride, tokens, d_topk_ids, d_topk_weights, d_out,
+                                 out_stride, d_workspace, workspace_bytes, stream);
+}
+
+extern "C" const float* aeon_moe_layer_logits(const aeon_moe_layer* layer, int tokens,
+                                              void* d_workspace) {
+    if (layer == nullptr || d_workspace == nullptr || tokens <= 0) return nullptr;
+    return carve(*layer, tokens, d_workspace).logits;
+}

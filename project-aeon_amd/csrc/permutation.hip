@@ -1,0 +1,148 @@
+// Token -> expert permutation (a stable counting sort of the (token, slot) draws by expert id)
+// and the segment list the decode kernels walk.
+//
+// Definition kept from the reference primitive: expert e owns positions
+// offsets[e] .. offsets[e+1); inside an expert the draws appear in ascending draw index, so the
+// placement is a pure function of the ids; an id outside [0, experts) is dropped.
+// Histogram + scan run in one workgroup (LDS atomics on integers, so the totals do not depend
+// on arrival order). The scatter gives every expert its own wave, which walks the draws in
+// order with ballot/popcount prefix sums: parallel across experts, sequential inside one, and
+// therefore deterministic without the O(experts x draws) single-thread walk.
+#include "permutation.hpp"
+
+namespace aeon355 {
+
+__device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
+#pragma unroll
+    for (int offset = 1; offset < 64; offset <<= 1) {
+        const int other = __shfl_up(v, offset, 64);
+        if (lane >= offset) v += other;
+    }
+    return v;
+}
+
+// Exclusive scan of one value per thread across a 1024-thread workgroup.
+__device__ __forceinline__ int block_exclusive_scan(int v, int* wave_totals, int* total) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int inclusive = wave_inclusive_scan(v, lane);
+    if (lane == 63) wave_totals[wave] = inclusive;
+    __syncthreads();
+    if (wave == 0) {
+        const int t = lane < 16 ? wave_totals[lane] : 0;
+        const int scanned = wave_inclusive_scan(t, lane);
+        if (lane < 16) wave_totals[lane] = scanned - t;
+        if (lane == 15) *total = scanned;
+    }
+    __syncthreads();
+    const int result = inclusive - v + wave_totals[wave];
+    __syncthreads();
+    return result;
+}
+
+__global__ __launch_bounds__(1024) void permutation_offsets_kernel(PermutationArgs a) {
+    __shared__ int histogram[kMaxPermutationExperts + 1];
+    __shared__ int wave_totals[16];
+    __shared__ int total;
+    const int lists = a.experts + (a.shared_tokens > 0 ? 1 : 0);
+    for (int e = threadIdx.x; e <= kMaxPermutationExperts; e += blockDim.x) histogram[e] = 0;
+    __syncthreads();
+    for (int d = threadIdx.x; d < a.draws; d += blockDim.x) {
+        const int e = a.ids[d];
+        if (e >= 0 && e < a.experts) atomicAdd(&histogram[e], 1);
+    }
+    if (threadIdx.x == 0 && a.shared_tokens > 0) histogram[a.experts] = a.shared_tokens;
+    __syncthreads();
+
+    const int e = threadIdx.x;
+    const int count = e < lists ? histogram[e] : 0;
+    const int offset = block_exclusive_scan(count, wave_totals, &total);
+    if (e < lists) a.offsets[e] = offset;
+    if (e == 0) a.offsets[lists] = total;
+
+    if (a.seg_expert != nullptr) {
+        const int segments = (count + a.seg_tokens - 1) / a.seg_tokens;
+        const int seg_base = block_exclusive_scan(segments, wave_totals, &total);
+        for (int s = 0; s < segments; ++s) {
+            const int at = seg_base + s;
+            if (at < a.seg_capacity) {
+                a.seg_expert[at] = e;
+                a.seg_first[at] = offset + s * a.seg_tokens;
+                a.seg_count[at] = min(a.seg_tokens, count - s * a.seg_tokens);
+            }
+        }
+        if (e == 0) *a.seg_total = min(total, a.seg_capacity);
+    }
+}
+
+// One wave per expert list; the list past the routed experts is the always-on expert, which
+// takes every token once, in token order, with weight 1 and its own output rows.
+__global__ __launch_bounds__(256) void permutation_scatter_kernel(PermutationArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int e = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lists = a.experts + (a.shared_tokens > 0 ? 1 : 0);
+    if (e >= lists) return;
+    int position = a.offsets[e];
+    const int end = a.offsets[e + 1];
+    if (position == end) return;
+    if (e == a.experts) {
+        for (int t = lane; t < a.shared_tokens; t += 64) {
+            a.token_indices[position + t] = t;
+            a.draw_indices[position + t] = a.draws + t;
+            if (a.weights_by_position != nullptr) a.weights_by_position[position + t] = 1.0f;
+        }
+        return;
+    }
+    for (int base = 0; base < a.draws && position < end; base += 64) {
+        const int d = base + lane;
+        const bool mine = d < a.draws && a.ids[d] == e;
+        const unsigned long long mask = __ballot(mine);
+        if (mine) {
+            const int at = position + __popcll(mask & ((1ull << lane) - 1ull));
+            a.token_indices[at] = d / a.slots;
+            a.draw_indices[at] = d;
+            if (a.weights_by_position != nullptr) a.weights_by_position[at] = a.weights_by_draw[d];
+        }
+        position += __popcll(mask);
+    }
+}
+
+int launch_permutation(const PermutationArgs& a, hipStream_t stream) {
+    permutation_offsets_kernel<<<1, 1024, 0, stream>>>(a);
+    AEON_LAUNCH_CHECK();
+    const int lists = a.experts + (a.shared_tokens > 0 ? 1 : 0);
+    permutation_scatter_kernel<<<(lists + 3) / 4, 256, 0, stream>>>(a);
+    AEON_LAUNCH_CHECK();
+    return AEON_OK;
+}
+
+}  // namespace aeon355
+
+using namespace aeon355;
+
+extern "C" int aeon_expert_permutation(const int32_t* d_topk_indices, int token_count, int slots,
+                                       int expert_count, int32_t* d_expert_offsets,
+                                       int32_t* d_token_indices, int32_t* d_draw_indices,
+                                       const float* d_weights_by_draw,
+                                       float* d_weights_by_position, void* stream) {
+    const char* who = "aeon_expert_permutation";
+    AEON_REQUIRE(d_topk_indices && d_expert_offsets && d_token_indices && d_draw_indices,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
+    AEON_REQUIRE(token_count >= 0 && slots > 0, AEON_ERR_INVALID_ARGUMENT, "%s: bad draw shape", who);
+    AEON_REQUIRE(expert_count > 0 && expert_count <= kMaxPermutationExperts,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: expert count out of range", who);
+    AEON_REQUIRE((d_weights_by_draw == nullptr) == (d_weights_by_position == nullptr),
+                 AEON_ERR_INVALID_ARGUMENT,
+                 "%s: weights need both a source and a destination", who);
+    PermutationArgs a{};
+    a.ids = d_topk_indices;
+    a.draws = token_count * slots;
+    a.slots = slots;
+    a.experts = expert_count;
+    a.offsets = d_expert_offsets;
+    a.token_indices = d_token_indices;
+    a.draw_indices = d_draw_indices;
+    a.weights_by_draw = d_weights_by_draw;
+    a.weights_by_position = d_weights_by_position;
+    return launch_permutation(a, as_stream(stream));
+}

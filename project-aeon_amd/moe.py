@@ -1,0 +1,153 @@
+"""Host-side view of the HBM-resident expert pool and of one MoE layer, over the C ABI.
+
+ExpertPool plays the part of the reference's UnifiedVRAMExpertPool
+(src/backend/swizzled_w4a16/core/vram_expert_pool.hpp:22-82): one device allocation cut into
+per-expert slots, each slot the six sub-tensors of an expert -- here in the wave64 packing, with
+every expert of the layer resident. torch is used for device memory and streams only.
+"""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import capi, synth
+
+CFG13 = (4, 8)
+CFG2 = (8, 4)
+
+
+class MoeLayerStruct(C.Structure):
+    _fields_ = [("hidden", C.c_int), ("intermediate", C.c_int), ("experts", C.c_int),
+                ("top_k", C.c_int), ("has_shared", C.c_int), ("swiglu_limit", C.c_float),
+                ("score_kind", C.c_int), ("routed_scaling_factor", C.c_float),
+                ("renormalize", C.c_int), ("d_router_weight", C.c_void_p),
+                ("d_router_bias", C.c_void_p), ("d_experts", C.c_void_p)]
+
+
+def stream_ptr():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+class ExpertPool:
+    """`slots` experts of shape (H, I) in the wave64 packing, 4096-byte aligned slots laid out
+    [W1 packed | W1 scale | W3 packed | W3 scale | W2 packed | W2 scale]."""
+
+    def __init__(self, slots, hidden, intermediate, device="cuda"):
+        self.slots, self.H, self.I = slots, hidden, intermediate
+        lib = capi.lib()
+        self.pb13 = lib.aeon_a64_packed_bytes(intermediate, hidden)
+        self.sb13 = lib.aeon_a64_scale_bytes(intermediate, hidden)
+        self.pb2 = lib.aeon_a64_packed_bytes(hidden, intermediate)
+        self.sb2 = lib.aeon_a64_scale_bytes(hidden, intermediate)
+        offs, at = [], 0
+        for b in (self.pb13, self.sb13, self.pb13, self.sb13, self.pb2, self.sb2):
+            offs.append(at)
+            at += (b + 255) // 256 * 256
+        self.offsets = offs
+        self.slot_bytes = (at + 4095) // 4096 * 4096
+        self.payload_bytes = 2 * (self.pb13 + self.sb13) + self.pb2 + self.sb2
+        self.buffer = torch.empty(slots * self.slot_bytes, dtype=torch.uint8, device=device)
+        base = self.buffer.data_ptr()
+        table = np.empty((slots, 6), dtype=np.int64)
+        for s in range(slots):
+            for j in range(6):
+                table[s, j] = base + s * self.slot_bytes + offs[j]
+        self.host_table = table
+        self.table = torch.from_numpy(table).to(device)
+
+    def expert_struct(self, slot):
+        return capi.A64Expert(*[int(v) for v in self.host_table[slot]])
+
+    def load_swizzled(self, slot, mats, mismatch=None):
+        """Load-time re-swizzle of one expert: `mats` = ((w1p, w1s), (w3p, w3s), (w2p, w2s)) device
+        tensors in the `.aeon` swizzled layout -> this slot's wave64 packing (device repack)."""
+        H, I = self.H, self.I
+        shapes = ((I, H, CFG13), (I, H, CFG13), (H, I, CFG2))
+        for j, ((p, s), (n, k, cfg)) in enumerate(zip(mats, shapes)):
+            capi.call("aeon_a64_repack_device", capi.vp(p), capi.vp(s), n, k, cfg[0], cfg[1],
+                      C.c_void_p(int(self.host_table[slot, 2 * j])),
+                      C.c_void_p(int(self.host_table[slot, 2 * j + 1])), capi.vp(mismatch),
+                      stream_ptr())
+
+    def fill_synthetic(self, seed, first_expert_id=0):
+        """Generate every slot on the device (`.aeon` layout, then the repack), expert id of slot
+        s = first_expert_id + s. Returns the number of 128-groups whose four group-32 scales
+        differed (must be 0)."""
+        H, I = self.H, self.I
+        dev = self.buffer.device
+        tmp = [(torch.empty(I * H // 2, dtype=torch.uint8, device=dev),
+                torch.empty(I * H // 32, dtype=torch.int16, device=dev)) for _ in range(2)]
+        tmp.append((torch.empty(H * I // 2, dtype=torch.uint8, device=dev),
+                    torch.empty(H * I // 32, dtype=torch.int16, device=dev)))
+        shapes = ((I, H, CFG13), (I, H, CFG13), (H, I, CFG2))
+        mismatch = torch.zeros(1, dtype=torch.int32, device=dev)
+        for s in range(self.slots):
+            for m, ((p, sc), (n, k, cfg)) in enumerate(zip(tmp, shapes)):
+                capi.call("aeon_synth_matrix_swizzled", C.c_uint64(seed), first_expert_id + s, m, n,
+                          k, cfg[0], cfg[1], capi.vp(p), capi.vp(sc), stream_ptr())
+            self.load_swizzled(s, tmp, mismatch)
+        return int(mismatch.item())
+
+
+class MoeLayer:
+    """One MoE layer: router + `experts` routed experts (+ an always-on shared expert held in
+    the pool's last slot)."""
+
+    def __init__(self, pool, experts, top_k, has_shared, swiglu_limit, router_weight=None,
+                 router_bias=None, score_kind=1, routed_scaling_factor=1.0, renormalize=True):
+        assert pool.slots == experts + (1 if has_shared else 0)
+        self.pool = pool
+        self.router_weight = router_weight
+        self.router_bias = router_bias
+        self.cfg = MoeLayerStruct(pool.H, pool.I, experts, top_k, int(has_shared), swiglu_limit,
+                                  score_kind, routed_scaling_factor, int(renormalize),
+                                  router_weight.data_ptr() if router_weight is not None else None,
+                                  router_bias.data_ptr() if router_bias is not None else None,
+                                  pool.table.data_ptr())
+        self.workspace = None
+        self.workspace_tokens = 0
+
+    def _workspace(self, tokens):
+        if self.workspace is None or tokens > self.workspace_tokens:
+            n = capi.lib().aeon_moe_layer_workspace_bytes(C.byref(self.cfg), tokens)
+            self.workspace = torch.empty(n, dtype=torch.uint8, device=self.pool.buffer.device)
+            self.workspace_tokens = tokens
+        return self.workspace
+
+    def decode(self, x, out=None, ids=None, weights=None):
+        """x fp16 [tokens][hidden] -> (out fp16 [tokens][hidden], ids int32, weights fp32)."""
+        tokens = x.shape[0]
+        ws = self._workspace(tokens)
+        k = self.cfg.top_k
+        out = torch.empty_like(x) if out is None else out
+        ids = torch.empty(tokens, k, dtype=torch.int32, device=x.device) if ids is None else ids
+        weights = (torch.empty(tokens, k, dtype=torch.float32, device=x.device)
+                   if weights is None else weights)
+        capi.call("aeon_moe_layer_decode", C.byref(self.cfg), capi.vp(x), x.stride(0), tokens,
+                  capi.vp(out), out.stride(0), capi.vp(ids), capi.vp(weights), capi.vp(ws),
+                  C.c_size_t(ws.numel()), stream_ptr())
+        return out, ids, weights
+
+    def routed(self, x, ids, weights, out=None):
+        """The expert part only, for given routing (ids int32 / weights fp32 [tokens][top_k])."""
+        tokens = x.shape[0]
+        ws = self._workspace(tokens)
+        out = torch.empty_like(x) if out is None else out
+        capi.call("aeon_moe_layer_routed", C.byref(self.cfg), capi.vp(x), x.stride(0), tokens,
+                  capi.vp(ids), capi.vp(weights), capi.vp(out), out.stride(0), capi.vp(ws),
+                  C.c_size_t(ws.numel()), stream_ptr())
+        return out
+
+    def router_logits(self, x):
+        """fp32 logits [tokens][experts] of x, by the same kernel (and so the same bits) the
+        decode step selects from."""
+        tokens = x.shape[0]
+        E = self.cfg.experts
+        lib = capi.lib()
+        n = lib.aeon_router_logits_workspace_bytes(tokens, self.cfg.hidden, E)
+        ws = torch.empty(max(n, 4), dtype=torch.uint8, device=x.device)
+        out = torch.empty(tokens, E, dtype=torch.float32, device=x.device)
+        capi.call("aeon_router_logits", capi.vp(x), x.stride(0), capi.vp(self.router_weight),
+                  capi.vp(out), tokens, self.cfg.hidden, E, capi.vp(ws), C.c_size_t(ws.numel()),
+                  stream_ptr())
+        return out

@@ -192,8 +192,9 @@ def test_swizzled_expert_trio_reference_shapes(orc, experts):
     assert h.rel_err(got_contrib, want_contrib) <= TOL
     # contrib == weight x unit-weight contribution, bit for bit (tests/test_v4_moe_accum_oracle.cpp)
     unit = torch.zeros_like(contrib)
+    ones = torch.ones(experts, device="cuda")
     capi.call("aeon_moe_fused_w2_contrib", capi.vp(hidden), C.byref(w2),
-              capi.vp(torch.ones(experts, device="cuda")), capi.vp(unit), experts, H, I, 8, 4,
+              capi.vp(ones), capi.vp(unit), experts, H, I, 8, 4,
               h.stream_ptr())
     assert torch.equal(contrib, unit * d_w[:, None])
     # fixed-order reduce: fp32 slot-order sum with the shared value as the initial term, one rounding

@@ -1,0 +1,190 @@
+"""GPU parity for the device-resident MoE layer: synthetic experts generated and re-swizzled on
+the device, router logits / top-k / permutation, and the full decode step of BASELINE config 2
+against the oracle."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+def _setup():
+    import torch
+    assert torch.cuda.is_available()
+    import helpers
+    from project_aeon_amd import capi, moe, synth
+    return torch, helpers, capi, moe, synth
+
+
+def test_device_generator_and_repack_bit_exact(orc):
+    """The device generator equals the host one, and the device repack equals the host repack,
+    for all three matrices of an expert at full size."""
+    torch, h, capi, moe, synth = _setup()
+    H, I = 7168, 2048
+    pool = moe.ExpertPool(2, H, I)
+    assert pool.fill_synthetic(seed=5, first_expert_id=40) == 0
+    torch.cuda.synchronize()
+    host = h.Expert(5, 41, H, I)
+    raw = pool.buffer.cpu().numpy()
+    base = pool.slot_bytes
+    for j, (m, which) in enumerate(((host.w1, "w1"), (host.w3, "w3"), (host.w2, "w2"))):
+        po, so = base + pool.offsets[2 * j], base + pool.offsets[2 * j + 1]
+        assert np.array_equal(raw[po:po + m.a64_packed.nbytes].view(np.uint32), m.a64_packed), which
+        assert np.array_equal(raw[so:so + m.a64_scale.nbytes].view(np.uint16), m.a64_scale), which
+    # the swizzled payload itself, for one matrix
+    p = torch.empty(I * H // 2, dtype=torch.uint8, device="cuda")
+    s = torch.empty(I * H // 32, dtype=torch.int16, device="cuda")
+    capi.call("aeon_synth_matrix_swizzled", C.c_uint64(5), 41, 1, I, H, 4, 8, capi.vp(p),
+              capi.vp(s), h.stream_ptr())
+    assert np.array_equal(p.cpu().numpy().view(np.uint32), host.w3.swz_packed)
+    assert np.array_equal(s.cpu().numpy().view(np.uint16), host.w3.swz_scale)
+
+
+def test_device_repack_flags_unequal_scales(orc):
+    torch, h, capi, moe, synth = _setup()
+    N, K = 32, 512
+    p, s128 = synth.expert_matrix_source(0, 0, 0, N, K)
+    s32 = np.ascontiguousarray(synth.scale32_from_scale128(s128)).view(np.uint16)
+    s32[7, 2] ^= 1
+    s32[9, 13] ^= 4
+    swp, sws = orc.swizzle(p, s32.ravel(), N, K, 4, 8)
+    out_p = torch.empty(N * K // 2, dtype=torch.uint8, device="cuda")
+    out_s = torch.empty(N * K // 128, dtype=torch.int16, device="cuda")
+    flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+    d_swp, d_sws = h.dev_u32(swp), h.dev_u16(sws)
+    capi.call("aeon_a64_repack_device", capi.vp(d_swp), capi.vp(d_sws), N, K, 4,
+              8, capi.vp(out_p), capi.vp(out_s), capi.vp(flag), h.stream_ptr())
+    assert int(flag.item()) == 2
+
+
+@pytest.mark.parametrize("score_kind,k,scaling", [(1, 8, 1.0), (0, 6, 1.5)])
+def test_router_ids_bit_exact_on_identical_logits(orc, score_kind, k, scaling):
+    torch, h, capi, moe, synth = _setup()
+    rng = np.random.default_rng(17)
+    T, E = 96, 256
+    logits = rng.normal(0, 2.0, (T, E)).astype(np.float32)
+    bias = rng.normal(0, 0.1, E).astype(np.float32)
+    # constructed ties: four experts share the top biased score (lowest index must win)
+    logits[0, [7, 40, 41, 200]] = 6.0
+    bias[[7, 40, 41, 200]] = 0.25
+    logits[1, :] = 0.5  # all equal up to the bias
+    d_ids = torch.zeros(T, k, dtype=torch.int32, device="cuda")
+    d_w = torch.zeros(T, k, dtype=torch.float32, device="cuda")
+    d_logits, d_bias = h.to_dev(logits), h.to_dev(bias)  # named: a temporary's memory is reused
+    capi.call("aeon_moe_router", capi.vp(d_logits), capi.vp(d_bias), None, None,
+              capi.vp(d_w), capi.vp(d_ids), T, E, k, C.c_float(scaling), 1, score_kind,
+              h.stream_ptr())
+    ids, w = d_ids.cpu().numpy(), d_w.cpu().numpy()
+    for t in range(T):
+        oi, ow = orc.router_topk(logits[t].astype(np.float64), bias.astype(np.float64), k, scaling,
+                                 score_kind)
+        assert np.array_equal(ids[t], oi), t
+        assert np.abs(w[t] - ow).max() <= 1e-5 * np.abs(ow).max()
+    assert list(ids[0][:4]) == [7, 40, 41, 200]
+    # bias-before-activation is a different (wrong) rule and must give a different selection somewhere
+    wrong = [orc.router_topk(logits[t].astype(np.float64), bias.astype(np.float64), k, scaling,
+                             score_kind, bias_before=True)[0] for t in range(T)]
+    assert any(not np.array_equal(ids[t], wrong[t]) for t in range(T))
+    # no bias, hash branch
+    table = rng.integers(0, E, (50, k)).astype(np.int64)
+    tok = rng.integers(0, 50, T).astype(np.int32)
+    d_table, d_tok = h.to_dev(table), h.to_dev(tok)
+    capi.call("aeon_moe_router", capi.vp(d_logits), None, capi.vp(d_table),
+              capi.vp(d_tok), capi.vp(d_w), capi.vp(d_ids), T, E, k, C.c_float(scaling), 1,
+              score_kind, h.stream_ptr())
+    ids = d_ids.cpu().numpy()
+    assert np.array_equal(ids, table[tok].astype(np.int32))
+
+
+@pytest.mark.parametrize("T,slots,E", [(1, 8, 256), (7, 6, 256), (300, 6, 256), (64, 8, 8),
+                                       (0, 8, 256), (2048, 8, 256), (64, 8, 1024)])
+def test_expert_permutation_bit_exact(orc, T, slots, E):
+    """Cases of tests/test_expert_permutation.cpp (T=1,7,300,64 at E=8, 0) plus the prefill size:
+    equality with the host stable counting sort, which implies the five invariants."""
+    torch, h, capi, moe, synth = _setup()
+    rng = np.random.default_rng(T * 31 + E)
+    ids = rng.integers(0, E, (T, slots)).astype(np.int32)
+    if T >= 7:
+        ids[3, 1] = -1      # out-of-range ids are dropped, not trusted
+        ids[5, 0] = E
+    wts = rng.random((T, slots)).astype(np.float32)
+    n = max(T * slots, 1)
+    d_off = torch.full((E + 1,), -7, dtype=torch.int32, device="cuda")
+    d_tok = torch.full((n,), -1, dtype=torch.int32, device="cuda")
+    d_drw = torch.full((n,), -1, dtype=torch.int32, device="cuda")
+    d_wp = torch.zeros(n, dtype=torch.float32, device="cuda")
+    d_ids = h.to_dev(ids.reshape(-1)) if T else d_tok
+    d_wd = h.to_dev(wts.reshape(-1)) if T else d_wp
+    capi.call("aeon_expert_permutation", capi.vp(d_ids), T, slots, E, capi.vp(d_off),
+              capi.vp(d_tok), capi.vp(d_drw), capi.vp(d_wd), capi.vp(d_wp), h.stream_ptr())
+    off, tok, drw = orc.expert_permutation(ids, T, slots, E)
+    assert np.array_equal(d_off.cpu().numpy(), off)
+    placed = int(off[E])
+    assert np.array_equal(d_tok.cpu().numpy()[:placed], tok[:placed])
+    assert np.array_equal(d_drw.cpu().numpy()[:placed], drw[:placed])
+    if placed:
+        assert np.array_equal(d_wp.cpu().numpy()[:placed], wts.reshape(-1)[drw[:placed]])
+
+
+def _oracle_layer(orc, h, experts, x, ids, weights, shared, limit):
+    """out[t] = half-rounded-shared + sum_k w_k * FFN_{id_k}(x_t), per the fixed-order combine,
+    with every FFN from the fp64 oracle (hidden rounded to fp16 as the device stores it)."""
+    T, k = ids.shape
+    H = x.shape[1]
+    contrib = np.zeros((T, k, H))
+    for e in np.unique(ids):
+        rows, slots = np.nonzero(ids == e)
+        o = experts[int(e)].ffn(x[rows], limit, round_hidden=True)
+        for i, (t, s) in enumerate(zip(rows, slots)):
+            contrib[t, s] = float(weights[t, s]) * o[i]
+    out = np.empty((T, H))
+    for t in range(T):
+        sh = None
+        if shared is not None:
+            sh = shared.ffn(x[t:t + 1], limit, round_hidden=True)[0].astype(np.float16).astype(np.float64)
+        out[t] = orc.moe_combine(contrib[t], sh)
+    return out
+
+
+@pytest.mark.parametrize("B", [1, 8, 32, 64])
+def test_config2_moe_layer_decode_reduced_experts(orc, B):
+    """BASELINE config 2 at full hidden/intermediate with a 24-expert layer (so the oracle can
+    regenerate every expert): fp32 router [7168 x E], sigmoid + bias, top-8, renormalised, one
+    always-on shared expert, int4 group-128 experts."""
+    torch, h, capi, moe, synth = _setup()
+    H, I, E, k, limit = 7168, 2048, 24, 8, 7.0
+    pool = moe.ExpertPool(E + 1, H, I)
+    assert pool.fill_synthetic(seed=2, first_expert_id=0) == 0
+    wr = synth.router_weight(2, H, E)
+    bias = synth.router_bias(2, E)
+    layer = moe.MoeLayer(pool, E, k, True, limit, h.to_dev(wr), h.to_dev(bias), score_kind=1)
+    x = synth.activations(2, B, H, unit=B)
+    d_x = h.dev_half(x)
+    out, ids, w = layer.decode(d_x)
+    logits = layer.router_logits(d_x).cpu().numpy()
+    torch.cuda.synchronize()
+    ids, w, out = ids.cpu().numpy(), w.cpu().numpy(), out.cpu().numpy()
+    # logits: fp32 device accumulation against the fp64 matvec
+    want_logits = x.astype(np.float64) @ wr.astype(np.float64)
+    assert np.abs(logits - want_logits).max() <= 1e-5 * np.abs(want_logits).max()
+    # ids / weights: the oracle on the device's own fp32 logits, bit-exact ids
+    for t in range(B):
+        oi, ow = orc.router_topk(logits[t].astype(np.float64), bias.astype(np.float64), k, 1.0, 1)
+        assert np.array_equal(ids[t], oi)
+        assert np.abs(w[t] - ow).max() <= 1e-5
+        assert abs(w[t].sum() - 1.0) < 1e-5
+    experts = {int(e): h.Expert(2, int(e), H, I) for e in np.unique(ids)}
+    shared = h.Expert(2, E, H, I)
+    want = _oracle_layer(orc, h, experts, x, ids, w, shared, limit)
+    assert np.abs(want).max() > 1.0
+    assert np.abs(out - want).max() <= 6e-3 * np.abs(want).max()
+    # routed-only entry point with the same routing gives the same bits
+    d_ids, d_w = h.to_dev(ids), h.to_dev(w)
+    again = layer.routed(d_x, d_ids, d_w)
+    assert np.array_equal(again.cpu().numpy(), out)
+    # and a run is bit-reproducible
+    out2, _, _ = layer.decode(d_x)
+    assert np.array_equal(out2.cpu().numpy(), out)
