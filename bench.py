@@ -1,0 +1,240 @@
+#!/usr/bin/env python3
+"""Benchmark of the routed-expert hot path on one MI355X.
+
+A "step" is one full MoE-layer decode (BASELINE config 2: fp32 router 7168x256 -> sigmoid+bias
+top-8 -> 256 int4 W4A16 experts + 1 always-on shared expert -> fixed-order weighted sum) over
+one batch of synthetic tokens, with every expert resident in HBM in the wave64 packing and all
+inputs already on the device when the timed region starts.
+
+Prints ONE JSON line: `value` = microseconds per token of the whole step; `roofline` = the
+dominant kernel (fused gate+up, which streams two of an expert's three matrices) against the
+8 TB/s HBM peak, timed live with events around repeated launches of that kernel alone;
+`cpu_baseline` = the CPU oracle (oracle/, a port of the reference's fp64 host oracle) on a
+bounded sample of the same batch, on this machine's host cores.
+"""
+import argparse
+import ctypes as C
+import importlib.util
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
+MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense fp16
+
+
+def _package():
+    if "project_aeon_amd" not in sys.modules:
+        pkg_dir = os.path.join(ROOT, "project-aeon_amd")
+        spec = importlib.util.spec_from_file_location(
+            "project_aeon_amd", os.path.join(pkg_dir, "__init__.py"),
+            submodule_search_locations=[pkg_dir])
+        module = importlib.util.module_from_spec(spec)
+        sys.modules["project_aeon_amd"] = module
+        spec.loader.exec_module(module)
+    return sys.modules["project_aeon_amd"]
+
+
+def matrix_bytes(n, k):
+    """Algorithmic bytes of one int4 matrix: packed nibbles + one fp16 scale per 128 columns."""
+    return n * k // 2 + n * (k // 128) * 2
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--batch", type=int, default=64, help="decode batch (1/8/32/64 in config 2)")
+    ap.add_argument("--experts", type=int, default=256)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
+    ap.add_argument("--cpu-tokens", type=int, default=4,
+                    help="tokens of the batch the CPU oracle is timed on")
+    ap.add_argument("--sweep", action="store_true",
+                    help="also report batch 1/8/32/64 in the `sweep` field")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU's share of the path; run with --gpus 1 "
+                 "(how the path would shard is described in DESIGN.md)")
+
+    import numpy as np
+    import torch
+
+    _package()
+    from project_aeon_amd import capi, moe, synth
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    capi.lib()
+    torch.cuda.set_device(0)
+    H, I, E, K_TOP, LIMIT, SEED = 7168, 2048, args.experts, 8, 7.0, 0
+    B = args.batch
+
+    t_setup = time.time()
+    pool = moe.ExpertPool(E + 1, H, I)
+    bad = pool.fill_synthetic(seed=SEED, first_expert_id=0)
+    assert bad == 0, "repack found group-32 scales that differ inside a 128-group"
+    wr = torch.from_numpy(synth.router_weight(SEED, H, E)).cuda()
+    bias = torch.from_numpy(synth.router_bias(SEED, E)).cuda()
+    layer = moe.MoeLayer(pool, E, K_TOP, True, LIMIT, wr, bias, score_kind=1)
+    torch.cuda.synchronize()
+    setup_s = time.time() - t_setup
+
+    def run_decode(batch, steps, warmup, rotate=8):
+        """Times `steps` layer steps; activations rotate over `rotate` seeded batches so the set
+        of routed experts changes from step to step."""
+        xs = [torch.from_numpy(synth.activations(SEED, batch, H, unit=1000 * batch + r)).cuda()
+              for r in range(rotate)]
+        out = torch.empty(batch, H, dtype=torch.float16, device="cuda")
+        ids = torch.empty(batch, K_TOP, dtype=torch.int32, device="cuda")
+        w = torch.empty(batch, K_TOP, dtype=torch.float32, device="cuda")
+        for i in range(warmup):
+            layer.decode(xs[i % rotate], out, ids, w)
+        torch.cuda.synchronize()
+        distinct = []
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        start.record()
+        for i in range(steps):
+            layer.decode(xs[i % rotate], out, ids, w)
+        stop.record()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+        ev_ms = start.elapsed_time(stop) / steps
+        for r in range(min(rotate, steps)):
+            layer.decode(xs[r], out, ids, w)
+            torch.cuda.synchronize()
+            distinct.append(int(torch.unique(ids).numel()))
+        d_mean = float(np.mean(distinct))
+        be = 3 * matrix_bytes(I, H)
+        step_bytes = (d_mean + 1) * be + H * E * 4 + batch * H * 2 * 2 + batch * K_TOP * 8
+        # dominant kernel alone: the state of the last full step is still in the workspace
+        x = xs[(min(rotate, steps) - 1)]
+        ws = layer._workspace(batch)
+
+        def gate_up_only():
+            capi.call("aeon_moe_layer_routed_stages", C.byref(layer.cfg), capi.vp(x), x.stride(0),
+                      batch, capi.vp(ids), capi.vp(w), capi.vp(out), out.stride(0), capi.vp(ws),
+                      C.c_size_t(ws.numel()), 2, moe.stream_ptr())
+
+        def down_only():
+            capi.call("aeon_moe_layer_routed_stages", C.byref(layer.cfg), capi.vp(x), x.stride(0),
+                      batch, capi.vp(ids), capi.vp(w), capi.vp(out), out.stride(0), capi.vp(ws),
+                      C.c_size_t(ws.numel()), 4, moe.stream_ptr())
+
+        def time_kernel(fn, reps):
+            fn()
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(reps):
+                fn()
+            b.record()
+            torch.cuda.synchronize()
+            return a.elapsed_time(b) / reps
+
+        reps = max(steps, 10)
+        gu_ms = time_kernel(gate_up_only, reps)
+        dn_ms = time_kernel(down_only, reps)
+        d_last = distinct[min(rotate, steps) - 1]
+        gu_bytes = (d_last + 1) * 2 * matrix_bytes(I, H) + batch * H * 2
+        dn_bytes = (d_last + 1) * matrix_bytes(H, I) + batch * (K_TOP + 1) * H * 4
+        return {
+            "batch": batch, "ms_per_step": ev_ms, "wall_ms_per_step": wall_ms,
+            "us_per_token": ev_ms * 1e3 / batch, "distinct_experts_mean": d_mean,
+            "step_bytes": step_bytes, "step_gbps": step_bytes / (ev_ms * 1e-3) / 1e9,
+            "gate_up_ms": gu_ms, "gate_up_bytes": gu_bytes,
+            "gate_up_gbps": gu_bytes / (gu_ms * 1e-3) / 1e9,
+            "down_ms": dn_ms, "down_bytes": dn_bytes, "down_gbps": dn_bytes / (dn_ms * 1e-3) / 1e9,
+            "x": x, "ids": ids.cpu().numpy(), "w": w.cpu().numpy(), "out": out.cpu().numpy(),
+        }
+
+    main_run = run_decode(B, args.steps, args.warmup)
+
+    sweep = None
+    if args.sweep:
+        sweep = []
+        for b in (1, 8, 32, 64):
+            r = main_run if b == B else run_decode(b, args.steps, args.warmup)
+            sweep.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()
+                          if k not in ("x", "ids", "w", "out")})
+
+    cpu = None
+    if not args.no_cpu:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        sys.path.insert(0, os.path.join(ROOT, "tests"))
+        import helpers
+        import orc
+        orc.lib()
+        n_tok = min(args.cpu_tokens, B)
+        x_host = main_run["x"][:n_tok].cpu().numpy()
+        ids_host, w_host = main_run["ids"][:n_tok], main_run["w"][:n_tok]
+        needed = sorted(set(int(e) for e in ids_host.ravel()) | {E})
+        experts = {e: helpers.Expert(SEED, e, H, I) for e in needed}   # untimed: input generation
+        threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        t0 = time.perf_counter()
+        # expert-major, one expert decoded at a time, fp64, OpenMP over output rows
+        contrib = np.zeros((n_tok, K_TOP, H))
+        for e in needed:
+            if e == E:
+                continue
+            rows, slots = np.nonzero(ids_host == e)
+            o = experts[e].ffn(x_host[rows], LIMIT, round_hidden=True)
+            for i, (t, s) in enumerate(zip(rows, slots)):
+                contrib[t, s] = float(w_host[t, s]) * o[i]
+        shared = experts[E].ffn(x_host, LIMIT, round_hidden=True)
+        ref_out = np.empty((n_tok, H))
+        for t in range(n_tok):
+            ref_out[t] = orc.moe_combine(contrib[t], shared[t].astype(np.float16).astype(np.float64))
+        cpu_s = time.perf_counter() - t0
+        err = float(np.abs(main_run["out"][:n_tok] - ref_out).max() / np.abs(ref_out).max())
+        cpu = {"value": round(cpu_s * 1e6 / n_tok, 1), "unit": "us/token", "cores": threads,
+               "kind": "port",
+               "sample": "first %d tokens of the batch-%d step, their %d distinct experts + the "
+                         "shared expert, expert-major fp64 oracle" % (n_tok, B, len(needed) - 1),
+               "gpu_vs_oracle_max_abs_over_peak": err}
+
+    result = {
+        "metric": "MoE-layer decode us/token",
+        "value": round(main_run["us_per_token"], 3),
+        "unit": "us/token",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(main_run["ms_per_step"], 4),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int4 weights x fp16 activations, fp32 accumulate",
+        "data": "synthetic (seeded int4 experts generated and re-swizzled on the device)",
+        "config": {"workload": "config2: full MoE layer decode, batch %d, hidden 7168, "
+                               "intermediate 2048, top-8 of %d experts + 1 shared, group-128 int4"
+                               % (B, E),
+                   "batch": B, "experts": E, "resident_expert_bytes": pool.payload_bytes * (E + 1),
+                   "distinct_routed_experts_per_step": round(main_run["distinct_experts_mean"], 1)},
+        "step_hbm": {"algorithmic_bytes": int(main_run["step_bytes"]),
+                     "achieved_gbps": round(main_run["step_gbps"], 1),
+                     "frac_of_peak": round(main_run["step_gbps"] / HBM_PEAK_GBPS, 4)},
+        "roofline": {"kernel": "a64_seg_kernel<gate_up> (fused W1+W3 dual-GEMV + clamped SwiGLU)",
+                     "bound": "hbm",
+                     "achieved": round(main_run["gate_up_gbps"], 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(main_run["gate_up_gbps"] / HBM_PEAK_GBPS, 4),
+                     "avg_launch_ms": round(main_run["gate_up_ms"], 4),
+                     "algorithmic_bytes": int(main_run["gate_up_bytes"]),
+                     "traffic": None},
+        "down_kernel": {"achieved_gbps": round(main_run["down_gbps"], 1),
+                        "avg_launch_ms": round(main_run["down_ms"], 4),
+                        "algorithmic_bytes": int(main_run["down_bytes"])},
+        "cpu_baseline": cpu,
+        "setup_s": round(setup_s, 1),
+    }
+    if sweep is not None:
+        result["sweep"] = sweep
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

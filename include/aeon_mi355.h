@@ -233,6 +233,20 @@ int aeon_moe_layer_routed(const aeon_moe_layer* layer, const void* d_x, int x_st
                           const int32_t* d_topk_ids, const float* d_topk_weights, void* d_out,
                           int out_stride, void* d_workspace, size_t workspace_bytes, void* stream);
 
+/* The same step cut into its launches, for measurement: runs only the stages named in
+ * stage_mask, on the state earlier stages left in the workspace (so AEON_STAGE_GATE_UP alone
+ * can be repeated between two events once a full step has run with the same arguments). */
+#define AEON_STAGE_PERMUTATION 1
+#define AEON_STAGE_GATE_UP 2
+#define AEON_STAGE_DOWN 4
+#define AEON_STAGE_REDUCE 8
+#define AEON_STAGE_ALL 15
+int aeon_moe_layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int x_stride,
+                                 int tokens, const int32_t* d_topk_ids,
+                                 const float* d_topk_weights, void* d_out, int out_stride,
+                                 void* d_workspace, size_t workspace_bytes, int stage_mask,
+                                 void* stream);
+
 /* Router + aeon_moe_layer_routed: the device half of run_layer_body_router
  * (v4_layer_body_moe.hpp:168-202) followed by run_layer_body_moe_and_post's expert part
  * (:285-312), with the per-layer D2H read-back and stream synchronisation of :188-192 removed.

@@ -89,11 +89,11 @@ extern "C" size_t aeon_moe_layer_workspace_bytes(const aeon_moe_layer* layer, in
     return carve(*layer, max_tokens, nullptr).bytes;
 }
 
-extern "C" int aeon_moe_layer_routed(const aeon_moe_layer* layer, const void* d_x, int x_stride,
-                                     int tokens, const int32_t* d_topk_ids,
-                                     const float* d_topk_weights, void* d_out, int out_stride,
-                                     void* d_workspace, size_t workspace_bytes, void* stream) {
-    const char* who = "aeon_moe_layer_routed";
+static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int x_stride,
+                               int tokens, const int32_t* d_topk_ids, const float* d_topk_weights,
+                               void* d_out, int out_stride, void* d_workspace,
+                               size_t workspace_bytes, int stage_mask, void* stream,
+                               const char* who) {
     if (int rc = check_layer(layer, who)) return rc;
     AEON_REQUIRE(d_x && d_topk_ids && d_topk_weights && d_out && d_workspace,
                  AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
@@ -125,7 +125,9 @@ extern "C" int aeon_moe_layer_routed(const aeon_moe_layer* layer, const void* d_
     p.seg_total = w.seg_total;
     p.seg_tokens = kSegTokens;
     p.seg_capacity = w.seg_capacity;
-    if (int rc = launch_permutation(p, s)) return rc;
+    if (stage_mask & AEON_STAGE_PERMUTATION) {
+        if (int rc = launch_permutation(p, s)) return rc;
+    }
 
     // Few live segments (a small batch) leave the chip idle unless K is also split.
     const int live_bound = (layer->has_shared ? (tokens + kSegTokens - 1) / kSegTokens : 0) +
@@ -143,7 +145,9 @@ extern "C" int aeon_moe_layer_routed(const aeon_moe_layer* layer, const void* d_
     gu.H = layer->hidden;
     gu.I = layer->intermediate;
     gu.limit = layer->swiglu_limit;
-    if (int rc = launch_seg_gate_up(gu, split_gate, s)) return rc;
+    if (stage_mask & AEON_STAGE_GATE_UP) {
+        if (int rc = launch_seg_gate_up(gu, split_gate, s)) return rc;
+    }
 
     SegDownArgs dn{};
     dn.hidden = w.hidden;
@@ -154,11 +158,32 @@ extern "C" int aeon_moe_layer_routed(const aeon_moe_layer* layer, const void* d_
     dn.contrib = w.contrib;
     dn.H = layer->hidden;
     dn.I = layer->intermediate;
-    if (int rc = launch_seg_down(dn, split_down, s)) return rc;
-
+    if (stage_mask & AEON_STAGE_DOWN) {
+        if (int rc = launch_seg_down(dn, split_down, s)) return rc;
+    }
+    if (!(stage_mask & AEON_STAGE_REDUCE)) return AEON_OK;
     return launch_token_reduce(w.contrib, tokens, layer->top_k, layer->has_shared ? draws : -1,
                                layer->has_shared ? nullptr : static_cast<const uint16_t*>(d_out),
                                out_stride, static_cast<uint16_t*>(d_out), out_stride, layer->hidden, s);
+}
+
+extern "C" int aeon_moe_layer_routed(const aeon_moe_layer* layer, const void* d_x, int x_stride,
+                                     int tokens, const int32_t* d_topk_ids,
+                                     const float* d_topk_weights, void* d_out, int out_stride,
+                                     void* d_workspace, size_t workspace_bytes, void* stream) {
+    return layer_routed_stages(layer, d_x, x_stride, tokens, d_topk_ids, d_topk_weights, d_out,
+                               out_stride, d_workspace, workspace_bytes, AEON_STAGE_ALL, stream,
+                               "aeon_moe_layer_routed");
+}
+
+extern "C" int aeon_moe_layer_routed_stages(const aeon_moe_layer* layer, const void* d_x,
+                                            int x_stride, int tokens, const int32_t* d_topk_ids,
+                                            const float* d_topk_weights, void* d_out,
+                                            int out_stride, void* d_workspace,
+                                            size_t workspace_bytes, int stage_mask, void* stream) {
+    return layer_routed_stages(layer, d_x, x_stride, tokens, d_topk_ids, d_topk_weights, d_out,
+                               out_stride, d_workspace, workspace_bytes, stage_mask, stream,
+                               "aeon_moe_layer_routed_stages");
 }
 
 extern "C" int aeon_moe_layer_decode(const aeon_moe_layer* layer, const void* d_x, int x_stride,
