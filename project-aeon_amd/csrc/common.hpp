@@ -48,7 +48,23 @@ typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
+
+// Pointers read out of a device-resident table are generic to the compiler, which then emits
+// FLAT loads (they count against both memory counters and cannot be waited on in order).
+// Every such pointer here is device global memory; saying so restores global_load and the
+// in-order vmcnt pipelining the kernels are written for.
+#define AEON_GLOBAL __attribute__((address_space(1)))
+template <class T>
+__device__ __forceinline__ const AEON_GLOBAL T* as_global(const T* p) {
+    return (const AEON_GLOBAL T*)(p);
+}
+template <class T>
+__device__ __forceinline__ const AEON_GLOBAL T* as_global(const void* p) {
+    return (const AEON_GLOBAL T*)(p);
+}
 
 union Word2Half {
     uint32_t u;
@@ -61,13 +77,22 @@ union Word2Half {
 // column 2j+1 in nibble 4+j, so masking with 0x000F000F yields the pair (2j, 2j+1) for j=0
 // directly. OR-ing 0x6400 makes the fp16 1024+q; a nibble left in bits 4..7 under 0x5400
 // reads as 64+q (the fp16 ulp at 64 is 1/16), which saves two of the four shifts.
+// (x & mask) | bits in one VALU instruction. The compiler emits v_and + v_or because a VOP3
+// instruction cannot carry two literals on this target; with the constants held in registers
+// the fused form applies.
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t bits) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(mask), "v"(bits));
+    return r;
+}
+
 __device__ __forceinline__ void unpack8(uint32_t w, half2_t out[4]) {
     Word2Half a, b, c, d;
     const uint32_t w8 = w >> 8;
-    a.u = (w & 0x000F000Fu) | 0x64006400u;
-    b.u = (w & 0x00F000F0u) | 0x54005400u;
-    c.u = (w8 & 0x000F000Fu) | 0x64006400u;
-    d.u = (w8 & 0x00F000F0u) | 0x54005400u;
+    a.u = and_or(w, 0x000F000Fu, 0x64006400u);
+    b.u = and_or(w, 0x00F000F0u, 0x54005400u);
+    c.u = and_or(w8, 0x000F000Fu, 0x64006400u);
+    d.u = and_or(w8, 0x00F000F0u, 0x54005400u);
     const half2_t k1032 = {(half_t)1032.0f, (half_t)1032.0f};
     const half2_t k72 = {(half_t)72.0f, (half_t)72.0f};
     out[0] = a.h - k1032;

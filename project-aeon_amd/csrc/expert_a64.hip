@@ -172,29 +172,29 @@ static int check_a64_shape(int N, int K, const char* who) {
 // MFMA segment kernels
 // ---------------------------------------------------------------------------------------------
 
-__device__ __forceinline__ float4_t mfma_group(const uint4& wq, const half8_t xf[4]) {
+__device__ __forceinline__ float4_t mfma_group(const u32x4_t& wq, const half8_t xf[4]) {
     float4_t t = {0.0f, 0.0f, 0.0f, 0.0f};
-    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(unpack8_vec(wq.x), xf[0], t, 0, 0, 0);
-    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(unpack8_vec(wq.y), xf[1], t, 0, 0, 0);
-    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(unpack8_vec(wq.z), xf[2], t, 0, 0, 0);
-    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(unpack8_vec(wq.w), xf[3], t, 0, 0, 0);
+    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(unpack8_vec(wq[0]), xf[0], t, 0, 0, 0);
+    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(unpack8_vec(wq[1]), xf[1], t, 0, 0, 0);
+    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(unpack8_vec(wq[2]), xf[2], t, 0, 0, 0);
+    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(unpack8_vec(wq[3]), xf[3], t, 0, 0, 0);
     return t;
 }
 
-__device__ __forceinline__ void scale_add(float4_t& acc, const float4_t& t, uint2 scale_bits) {
-    acc[0] += half_bits_to_float(static_cast<uint16_t>(scale_bits.x & 0xFFFFu)) * t[0];
-    acc[1] += half_bits_to_float(static_cast<uint16_t>(scale_bits.x >> 16)) * t[1];
-    acc[2] += half_bits_to_float(static_cast<uint16_t>(scale_bits.y & 0xFFFFu)) * t[2];
-    acc[3] += half_bits_to_float(static_cast<uint16_t>(scale_bits.y >> 16)) * t[3];
+__device__ __forceinline__ void scale_add(float4_t& acc, const float4_t& t, u32x2_t scale_bits) {
+    acc[0] += half_bits_to_float(static_cast<uint16_t>(scale_bits[0] & 0xFFFFu)) * t[0];
+    acc[1] += half_bits_to_float(static_cast<uint16_t>(scale_bits[0] >> 16)) * t[1];
+    acc[2] += half_bits_to_float(static_cast<uint16_t>(scale_bits[1] & 0xFFFFu)) * t[2];
+    acc[3] += half_bits_to_float(static_cast<uint16_t>(scale_bits[1] >> 16)) * t[3];
 }
 
-constexpr int kSegPrefetch = 2;  // 128-column groups per wave per step
-
-// One workgroup = one (16-row tile, segment). Lane l supplies weight row l%16 / token l%16 and
-// the 8-column chunk l/16 of each 32-column MFMA step; it ends up holding output rows
-// 4*(l/16)..+3 of token l%16.
-template <bool GATE_UP, int WK>
+// One workgroup = (R consecutive 16-row tiles, one segment). Lane l supplies weight row l%16 of
+// each tile / token l%16 and the 8-column chunk l/16 of each 32-column MFMA step; it ends up
+// holding output rows 4*(l/16)..+3 of token l%16 for each tile. The activation fragments of a
+// 128-column group are loaded once and used by all R tiles (and both matrices of gate/up).
+template <bool GATE_UP, int R, int WK, int D>
 __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegDownArgs dn) {
+    constexpr int NM = GATE_UP ? 2 : 1;
     const SegmentList& seg = GATE_UP ? gu.seg : dn.seg;
     const int s = blockIdx.y;
     int first = 0;
@@ -211,123 +211,341 @@ __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegD
     const int wave = threadIdx.x >> 6;
     const int n = lane & 15;
     const int chunk = lane >> 4;
-    const int tile = blockIdx.x;
+    const int tile0 = blockIdx.x * R;
 
     const int K = GATE_UP ? gu.H : dn.I;
     const int groups = K / 128;
-    const uint4* pa = static_cast<const uint4*>(GATE_UP ? e.w1_packed : e.w2_packed);
-    const uint16_t* sa = static_cast<const uint16_t*>(GATE_UP ? e.w1_scale : e.w2_scale);
-    const uint4* pb = static_cast<const uint4*>(e.w3_packed);
-    const uint16_t* sb = static_cast<const uint16_t*>(e.w3_scale);
+    const AEON_GLOBAL u32x4_t* pm[NM];
+    const AEON_GLOBAL uint16_t* sm[NM];
+    pm[0] = as_global<u32x4_t>(GATE_UP ? e.w1_packed : e.w2_packed);
+    sm[0] = as_global<uint16_t>(GATE_UP ? e.w1_scale : e.w2_scale);
+    if (GATE_UP) {
+        pm[NM - 1] = as_global<u32x4_t>(e.w3_packed);
+        sm[NM - 1] = as_global<uint16_t>(e.w3_scale);
+    }
 
     // A padded token column repeats the segment's last live position: always a valid row, and
     // its products land in output columns the store below never writes.
     const int position = first + (n < count ? n : count - 1);
-    const uint16_t* xrow;
+    const AEON_GLOBAL uint16_t* xrow;
     if (GATE_UP) {
         const long row = gu.row_index != nullptr ? gu.row_index[position] : position;
-        xrow = gu.x + row * gu.x_stride + chunk * 8;
+        xrow = as_global<uint16_t>(gu.x) + row * gu.x_stride + chunk * 8;
     } else {
-        xrow = dn.hidden + static_cast<size_t>(position) * dn.I + chunk * 8;
+        xrow = as_global<uint16_t>(dn.hidden) + static_cast<size_t>(position) * dn.I + chunk * 8;
     }
 
-    const size_t tile_base = static_cast<size_t>(tile) * groups;
-    float4_t acc_a = {0.0f, 0.0f, 0.0f, 0.0f};
-    float4_t acc_b = {0.0f, 0.0f, 0.0f, 0.0f};
+    float4_t acc[NM][R];
+#pragma unroll
+    for (int m = 0; m < NM; ++m)
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[m][r] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-    for (int g0 = wave; g0 < groups; g0 += WK * kSegPrefetch) {
-        uint4 wa[kSegPrefetch], wb[kSegPrefetch];
-        uint2 ca[kSegPrefetch], cb[kSegPrefetch];
-        half8_t xf[kSegPrefetch][4];
+    // Software pipeline over the 128-column groups this wave owns (g = wave, wave+WK, ...):
+    // D groups of weights, scales and activation fragments are in flight in registers; a
+    // buffer is refilled for the group D steps ahead as soon as its MFMAs have been issued, so
+    // every wave keeps D*NM*R KiB of HBM reads outstanding while it computes.
+    u32x4_t wq[D][NM][R];
+    u32x2_t sc[D][NM][R];
+    half8_t xf[D][4];
+    auto load_group = [&](int d, int g) {
 #pragma unroll
-        for (int j = 0; j < kSegPrefetch; ++j) {
-            const int g = g0 + j * WK;
-            if (g < groups) {
-                wa[j] = pa[(tile_base + g) * 64 + lane];
-                ca[j] = *reinterpret_cast<const uint2*>(sa + (tile_base + g) * 16 + chunk * 4);
-                if (GATE_UP) {
-                    wb[j] = pb[(tile_base + g) * 64 + lane];
-                    cb[j] = *reinterpret_cast<const uint2*>(sb + (tile_base + g) * 16 + chunk * 4);
-                }
+        for (int m = 0; m < NM; ++m)
 #pragma unroll
-                for (int st = 0; st < 4; ++st) {
-                    xf[j][st] = *reinterpret_cast<const half8_t*>(xrow + g * 128 + st * 32);
-                }
+            for (int r = 0; r < R; ++r) {
+                const size_t t = static_cast<size_t>(tile0 + r) * groups + g;
+                wq[d][m][r] = pm[m][t * 64 + lane];
+                sc[d][m][r] = *reinterpret_cast<const AEON_GLOBAL u32x2_t*>(sm[m] + t * 16 + chunk * 4);
             }
-        }
 #pragma unroll
-        for (int j = 0; j < kSegPrefetch; ++j) {
-            const int g = g0 + j * WK;
-            if (g < groups) {
-                scale_add(acc_a, mfma_group(wa[j], xf[j]), ca[j]);
-                if (GATE_UP) scale_add(acc_b, mfma_group(wb[j], xf[j]), cb[j]);
-            }
+        for (int st = 0; st < 4; ++st) {
+            xf[d][st] = *reinterpret_cast<const AEON_GLOBAL half8_t*>(xrow + g * 128 + st * 32);
         }
+    };
+    // Group j of this wave is column group wave + j*WK; it owns `mine` of them. The loop is cut
+    // in three so that the steady state has no conditional loads: a branch around a prefetch
+    // makes the compiler wait for every outstanding load at the loop head (the two paths leave
+    // different numbers in flight), which would serialise the pipeline.
+    const int mine = (groups - wave + WK - 1) / WK;
+    auto compute = [&](int d) {
+#pragma unroll
+        for (int m = 0; m < NM; ++m)
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                scale_add(acc[m][r], mfma_group(wq[d][m][r], xf[d]), sc[d][m][r]);
+            }
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        const int j = d < mine ? d : mine - 1;  // a short wave reloads its last group, unused
+        load_group(d, wave + j * WK);
+    }
+    int j0 = 0;
+    for (; j0 + 2 * D <= mine; j0 += D) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            compute(d);
+            load_group(d, wave + (j0 + d + D) * WK);
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        if (j0 + d < mine) {
+            compute(d);
+            if (j0 + d + D < mine) load_group(d, wave + (j0 + d + D) * WK);
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        if (j0 + D + d < mine) compute(d);
     }
 
     if (WK > 1) {
-        __shared__ float4_t partial[WK][2][64];
-        partial[wave][0][lane] = acc_a;
-        if (GATE_UP) partial[wave][1][lane] = acc_b;
+        __shared__ float4_t partial[WK][NM][R][64];
+#pragma unroll
+        for (int m = 0; m < NM; ++m)
+#pragma unroll
+            for (int r = 0; r < R; ++r) partial[wave][m][r][lane] = acc[m][r];
         __syncthreads();
         if (wave != 0) return;
 #pragma unroll
-        for (int w = 1; w < WK; ++w) {
-            acc_a += partial[w][0][lane];
-            if (GATE_UP) acc_b += partial[w][1][lane];
-        }
+        for (int w = 1; w < WK; ++w)
+#pragma unroll
+            for (int m = 0; m < NM; ++m)
+#pragma unroll
+                for (int r = 0; r < R; ++r) acc[m][r] += partial[w][m][r][lane];
     }
 
     if (n >= count) return;
-    const int row0 = tile * 16 + chunk * 4;
-    if (GATE_UP) {
-        uint2 packed;
-        packed.x = float_to_half_bits(clamped_swiglu(acc_a[0], acc_b[0], gu.limit)) |
-                   (static_cast<uint32_t>(float_to_half_bits(
-                        clamped_swiglu(acc_a[1], acc_b[1], gu.limit))) << 16);
-        packed.y = float_to_half_bits(clamped_swiglu(acc_a[2], acc_b[2], gu.limit)) |
-                   (static_cast<uint32_t>(float_to_half_bits(
-                        clamped_swiglu(acc_a[3], acc_b[3], gu.limit))) << 16);
-        *reinterpret_cast<uint2*>(gu.hidden + static_cast<size_t>(first + n) * gu.I + row0) = packed;
-    } else {
-        const float w = dn.weight[first + n];
-        const float4_t v = {w * acc_a[0], w * acc_a[1], w * acc_a[2], w * acc_a[3]};
-        const size_t out_row = dn.out_row != nullptr ? dn.out_row[first + n] : first + n;
-        *reinterpret_cast<float4_t*>(dn.contrib + out_row * dn.H + row0) = v;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int row0 = (tile0 + r) * 16 + chunk * 4;
+        if (GATE_UP) {
+            const float4_t& ga = acc[0][r];
+            const float4_t& up = acc[NM - 1][r];
+            uint2 packed;
+            packed.x = float_to_half_bits(clamped_swiglu(ga[0], up[0], gu.limit)) |
+                       (static_cast<uint32_t>(float_to_half_bits(
+                            clamped_swiglu(ga[1], up[1], gu.limit))) << 16);
+            packed.y = float_to_half_bits(clamped_swiglu(ga[2], up[2], gu.limit)) |
+                       (static_cast<uint32_t>(float_to_half_bits(
+                            clamped_swiglu(ga[3], up[3], gu.limit))) << 16);
+            *reinterpret_cast<uint2*>(gu.hidden + static_cast<size_t>(first + n) * gu.I + row0) = packed;
+        } else {
+            const float w = dn.weight[first + n];
+            const float4_t v = {w * acc[0][r][0], w * acc[0][r][1], w * acc[0][r][2], w * acc[0][r][3]};
+            const size_t out_row = dn.out_row != nullptr ? dn.out_row[first + n] : first + n;
+            *reinterpret_cast<float4_t*>(dn.contrib + out_row * dn.H + row0) = v;
+        }
     }
 }
 
-int launch_seg_gate_up(const SegGateUpArgs& a, int k_split, hipStream_t stream) {
+// The wide form for steps with many live segments: four waves per workgroup, each with its own
+// R tiles and no K split. What limits the narrow form is the number of vector-memory
+// instructions per weight byte (each wave issues 4 activation and NM*R scale loads beside its
+// NM*R weight loads for every 128 columns), so this form takes both off that pipe:
+//   * the scales of a wave's tiles (groups x 32 bytes each, contiguous) are copied into LDS
+//     once, before the loop, and read back with one ds_read_b64 per tile and group;
+//   * the four waves share one copy of the segment's activation fragments: per group every
+//     wave fetches one fragment (16 tokens x 32 columns) and all four read them from LDS.
+// Per wave and group that leaves NM*R weight loads + 1 activation load.
+template <bool GATE_UP, int R, int D>
+__global__ __launch_bounds__(256) void a64_seg_wide_kernel(SegGateUpArgs gu, SegDownArgs dn) {
+    constexpr int NM = GATE_UP ? 2 : 1;
+    const SegmentList& seg = GATE_UP ? gu.seg : dn.seg;
+    const int s = blockIdx.y;
+    if (s >= *seg.total) return;
+    const int first = seg.first[s];
+    const int count = seg.count[s];
+    const aeon_a64_expert e = (GATE_UP ? gu.experts : dn.experts)[seg.expert[s]];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int n = lane & 15;
+    const int chunk = lane >> 4;
+    const int tile0 = (blockIdx.x * 4 + wave) * R;
+
+    const int K = GATE_UP ? gu.H : dn.I;
+    const int groups = K / 128;
+    const AEON_GLOBAL u32x4_t* pm[NM];
+    const AEON_GLOBAL uint16_t* sm[NM];
+    pm[0] = as_global<u32x4_t>(GATE_UP ? e.w1_packed : e.w2_packed);
+    sm[0] = as_global<uint16_t>(GATE_UP ? e.w1_scale : e.w2_scale);
+    if (GATE_UP) {
+        pm[NM - 1] = as_global<u32x4_t>(e.w3_packed);
+        sm[NM - 1] = as_global<uint16_t>(e.w3_scale);
+    }
+
+    const int position = first + (n < count ? n : count - 1);
+    const AEON_GLOBAL uint16_t* xrow;
+    if (GATE_UP) {
+        const long row = gu.row_index != nullptr ? gu.row_index[position] : position;
+        xrow = as_global<uint16_t>(gu.x) + row * gu.x_stride + chunk * 8;
+    } else {
+        xrow = as_global<uint16_t>(dn.hidden) + static_cast<size_t>(position) * dn.I + chunk * 8;
+    }
+    // this wave's share of a group's activations: MFMA step `wave` (columns 32*wave..+31)
+    xrow += wave * 32;
+
+    __shared__ half8_t xs[2][4][64];
+    extern __shared__ u32x4_t scale_lds[];  // [wave][m][r][groups * 2] 16-byte units
+    const int tile_u4 = groups * 2;         // 32 bytes of scales per group
+    u32x4_t* my_scales = scale_lds + static_cast<size_t>(wave) * NM * R * tile_u4;
+#pragma unroll
+    for (int m = 0; m < NM; ++m)
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const AEON_GLOBAL u32x4_t* src = reinterpret_cast<const AEON_GLOBAL u32x4_t*>(
+                sm[m] + static_cast<size_t>(tile0 + r) * groups * 16);
+            for (int i = lane; i < tile_u4; i += 64) my_scales[(m * R + r) * tile_u4 + i] = src[i];
+        }
+
+    float4_t acc[NM][R];
+#pragma unroll
+    for (int m = 0; m < NM; ++m)
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[m][r] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+    u32x4_t wq[D][NM][R];
+    auto load_group = [&](int d, int g) {
+#pragma unroll
+        for (int m = 0; m < NM; ++m)
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const size_t t = static_cast<size_t>(tile0 + r) * groups + g;
+                wq[d][m][r] = pm[m][t * 64 + lane];
+            }
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d) load_group(d, d < groups ? d : groups - 1);
+    xs[0][wave][lane] = *reinterpret_cast<const AEON_GLOBAL half8_t*>(xrow);
+    __syncthreads();
+
+    // step g: fetch this wave's fragment of group g+1, read all four fragments of group g from
+    // LDS, multiply, then publish the fetched fragment into the other LDS buffer. One barrier
+    // per group: buffer (g+1)&1 was last read in step g-1, before that step's barrier.
+    const u32x2_t* scale_rows = reinterpret_cast<const u32x2_t*>(my_scales) + chunk;
+    auto step = [&](int d, int g, bool refill) {
+        const int gx = g + 1 < groups ? g + 1 : g;  // the last step refetches its own group, unused
+        const half8_t xnext = *reinterpret_cast<const AEON_GLOBAL half8_t*>(xrow + gx * 128);
+        half8_t xf[4];
+#pragma unroll
+        for (int st = 0; st < 4; ++st) xf[st] = xs[g & 1][st][lane];
+#pragma unroll
+        for (int m = 0; m < NM; ++m)
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                // scales of (tile, group): 16 rows x 2 bytes; this lane's rows are 4*chunk..+3
+                const u32x2_t sc = scale_rows[((m * R + r) * tile_u4 + g * 2) * 2];
+                scale_add(acc[m][r], mfma_group(wq[d][m][r], xf), sc);
+            }
+        if (refill) load_group(d, g + D);
+        xs[(g + 1) & 1][wave][lane] = xnext;
+        __syncthreads();
+    };
+    int g0 = 0;
+    for (; g0 + 2 * D <= groups; g0 += D) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) step(d, g0 + d, true);
+    }
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        if (g0 + d < groups) step(d, g0 + d, g0 + d + D < groups);
+    }
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        if (g0 + D + d < groups) step(d, g0 + D + d, false);
+    }
+
+    if (n >= count) return;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int row0 = (tile0 + r) * 16 + chunk * 4;
+        if (GATE_UP) {
+            const float4_t& ga = acc[0][r];
+            const float4_t& up = acc[NM - 1][r];
+            uint2 packed;
+            packed.x = float_to_half_bits(clamped_swiglu(ga[0], up[0], gu.limit)) |
+                       (static_cast<uint32_t>(float_to_half_bits(
+                            clamped_swiglu(ga[1], up[1], gu.limit))) << 16);
+            packed.y = float_to_half_bits(clamped_swiglu(ga[2], up[2], gu.limit)) |
+                       (static_cast<uint32_t>(float_to_half_bits(
+                            clamped_swiglu(ga[3], up[3], gu.limit))) << 16);
+            *reinterpret_cast<uint2*>(gu.hidden + static_cast<size_t>(first + n) * gu.I + row0) = packed;
+        } else {
+            const float w = dn.weight[first + n];
+            const float4_t v = {w * acc[0][r][0], w * acc[0][r][1], w * acc[0][r][2], w * acc[0][r][3]};
+            const size_t out_row = dn.out_row != nullptr ? dn.out_row[first + n] : first + n;
+            *reinterpret_cast<float4_t*>(dn.contrib + out_row * dn.H + row0) = v;
+        }
+    }
+}
+
+int g_seg_depth = 2;  // measurement override of the pipeline depth
+
+template <bool GATE_UP, int R, int D>
+static void launch_seg_rd(const SegGateUpArgs& gu, const SegDownArgs& dn, int tiles, int capacity,
+                          int k_split, hipStream_t stream) {
+    const dim3 grid(tiles / R, capacity);
+    if (k_split == 0) {
+        const int k_dim = GATE_UP ? gu.H : dn.I;
+        const size_t scale_bytes = static_cast<size_t>(4) * (GATE_UP ? 2 : 1) * R * (k_dim / 128) * 32;
+        a64_seg_wide_kernel<GATE_UP, R, D>
+            <<<dim3(tiles / (4 * R), capacity), 256, scale_bytes, stream>>>(gu, dn);
+    } else if (k_split >= 4) {
+        a64_seg_kernel<GATE_UP, R, 4, D><<<grid, 256, 0, stream>>>(gu, dn);
+    } else if (k_split == 2) {
+        a64_seg_kernel<GATE_UP, R, 2, D><<<grid, 128, 0, stream>>>(gu, dn);
+    } else {
+        a64_seg_kernel<GATE_UP, R, 1, D><<<grid, 64, 0, stream>>>(gu, dn);
+    }
+}
+
+template <bool GATE_UP, int R>
+static void launch_seg_r(const SegGateUpArgs& gu, const SegDownArgs& dn, int tiles, int capacity,
+                         int k_split, hipStream_t stream) {
+    if (g_seg_depth >= 4) {
+        launch_seg_rd<GATE_UP, R, 4>(gu, dn, tiles, capacity, k_split, stream);
+    } else if (g_seg_depth == 3) {
+        launch_seg_rd<GATE_UP, R, 3>(gu, dn, tiles, capacity, k_split, stream);
+    } else if (g_seg_depth == 2) {
+        launch_seg_rd<GATE_UP, R, 2>(gu, dn, tiles, capacity, k_split, stream);
+    } else {
+        launch_seg_rd<GATE_UP, R, 1>(gu, dn, tiles, capacity, k_split, stream);
+    }
+}
+
+template <bool GATE_UP>
+static void launch_seg(const SegGateUpArgs& gu, const SegDownArgs& dn, int tiles, int capacity,
+                       int k_split, int row_tiles, hipStream_t stream) {
+    const bool direct = (GATE_UP ? gu.seg.total : dn.seg.total) == nullptr;
+    if (k_split == 0 && (direct || tiles % (4 * (row_tiles >= 4 ? 4 : row_tiles >= 2 ? 2 : 1)) != 0)) {
+        k_split = 1;  // the wide form needs a segment list and whole workgroups of tiles
+    }
+    if (row_tiles >= 4 && tiles % 4 == 0) {
+        launch_seg_r<GATE_UP, 4>(gu, dn, tiles, capacity, k_split, stream);
+    } else if (row_tiles >= 2 && tiles % 2 == 0) {
+        launch_seg_r<GATE_UP, 2>(gu, dn, tiles, capacity, k_split, stream);
+    } else {
+        launch_seg_r<GATE_UP, 1>(gu, dn, tiles, capacity, k_split, stream);
+    }
+}
+
+int launch_seg_gate_up(const SegGateUpArgs& a, int k_split, int row_tiles, hipStream_t stream) {
     AEON_REQUIRE(a.H % 128 == 0 && a.I % 16 == 0 && a.x_stride % 8 == 0, AEON_ERR_INVALID_ARGUMENT,
                  "gate/up segments: need H%%128==0, I%%16==0 and an activation pitch that keeps "
                  "rows 16-byte aligned (H=%d I=%d pitch=%ld)", a.H, a.I, a.x_stride);
     if (a.seg.capacity <= 0) return AEON_OK;
-    const dim3 grid(a.I / 16, a.seg.capacity);
-    const SegDownArgs none{};
-    if (k_split >= 4) {
-        a64_seg_kernel<true, 4><<<grid, 256, 0, stream>>>(a, none);
-    } else if (k_split == 2) {
-        a64_seg_kernel<true, 2><<<grid, 128, 0, stream>>>(a, none);
-    } else {
-        a64_seg_kernel<true, 1><<<grid, 64, 0, stream>>>(a, none);
-    }
+    launch_seg<true>(a, SegDownArgs{}, a.I / 16, a.seg.capacity, k_split, row_tiles, stream);
     AEON_LAUNCH_CHECK();
     return AEON_OK;
 }
 
-int launch_seg_down(const SegDownArgs& a, int k_split, hipStream_t stream) {
+int launch_seg_down(const SegDownArgs& a, int k_split, int row_tiles, hipStream_t stream) {
     AEON_REQUIRE(a.I % 128 == 0 && a.H % 16 == 0, AEON_ERR_INVALID_ARGUMENT,
                  "down segments: need I%%128==0 and H%%16==0 (H=%d I=%d)", a.H, a.I);
     if (a.seg.capacity <= 0) return AEON_OK;
-    const dim3 grid(a.H / 16, a.seg.capacity);
-    const SegGateUpArgs none{};
-    if (k_split >= 4) {
-        a64_seg_kernel<false, 4><<<grid, 256, 0, stream>>>(none, a);
-    } else if (k_split == 2) {
-        a64_seg_kernel<false, 2><<<grid, 128, 0, stream>>>(none, a);
-    } else {
-        a64_seg_kernel<false, 1><<<grid, 64, 0, stream>>>(none, a);
-    }
+    launch_seg<false>(SegGateUpArgs{}, a, a.H / 16, a.seg.capacity, k_split, row_tiles, stream);
     AEON_LAUNCH_CHECK();
     return AEON_OK;
 }
@@ -448,7 +666,7 @@ extern "C" int aeon_a64_expert_decode(const void* d_x, int tokens, const aeon_a6
         gu.seg.capacity = 1;
         gu.direct_expert = *expert;
         gu.direct_count = tokens;
-        if (int rc = launch_seg_gate_up(gu, 4, s)) return rc;
+        if (int rc = launch_seg_gate_up(gu, 4, 1, s)) return rc;
         SegDownArgs dn{};
         dn.hidden = static_cast<const uint16_t*>(d_hidden);
         dn.weight = d_route_weights;
@@ -458,7 +676,7 @@ extern "C" int aeon_a64_expert_decode(const void* d_x, int tokens, const aeon_a6
         dn.seg.capacity = 1;
         dn.direct_expert = *expert;
         dn.direct_count = tokens;
-        if (int rc = launch_seg_down(dn, 4, s)) return rc;
+        if (int rc = launch_seg_down(dn, 4, 1, s)) return rc;
     } else {
         GemvArgs g{};
         g.x = static_cast<const uint16_t*>(d_x);

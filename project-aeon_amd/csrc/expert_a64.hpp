@@ -44,9 +44,12 @@ struct SegDownArgs {
     int direct_count;
 };
 
-// k_split: 1, 2 or 4 waves of a workgroup share one 16-row tile and split K between them.
-int launch_seg_gate_up(const SegGateUpArgs& a, int k_split, hipStream_t stream);
-int launch_seg_down(const SegDownArgs& a, int k_split, hipStream_t stream);
+// k_split: 1, 2 or 4 waves of a workgroup split K between them. row_tiles: 1, 2 or 4
+// consecutive 16-row tiles per workgroup share one read of the activations.
+int launch_seg_gate_up(const SegGateUpArgs& a, int k_split, int row_tiles, hipStream_t stream);
+int launch_seg_down(const SegDownArgs& a, int k_split, int row_tiles, hipStream_t stream);
+
+extern int g_seg_depth;
 
 // out[t][i] = half( [shared: float(half(contrib[shared_base + t][i]))] +
 //                   sum_{s < slots, ascending} contrib[t*slots + s][i] ),

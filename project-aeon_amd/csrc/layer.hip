@@ -6,6 +6,8 @@
 #include "expert_a64.hpp"
 #include "permutation.hpp"
 
+#include <cstdlib>
+
 extern "C" size_t aeon_router_logits_workspace_bytes(int tokens, int hidden, int experts);
 
 namespace aeon355 {
@@ -132,8 +134,15 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     // Few live segments (a small batch) leave the chip idle unless K is also split.
     const int live_bound = (layer->has_shared ? (tokens + kSegTokens - 1) / kSegTokens : 0) +
                            (draws < layer->experts ? draws : layer->experts);
-    const int split_gate = live_bound * (layer->intermediate / 16) >= 8192 ? 1 : 4;
-    const int split_down = live_bound * (layer->hidden / 16) >= 8192 ? 1 : 4;
+    // Many live segments: the wide kernels (k_split 0: four waves per workgroup sharing the
+    // activations through LDS, no K split). Few: split K four ways so the chip still fills.
+    int split_gate = live_bound * (layer->intermediate / 16) >= 8192 ? 0 : 4;
+    int split_down = live_bound * (layer->hidden / 16) >= 8192 ? 0 : 4;
+    int rows_gate = split_gate == 0 ? 2 : 1;
+    int rows_down = split_down == 0 ? 4 : 1;
+    if (const char* t = getenv("AEON_TUNE")) {  // "kg rg kd rd": measurement override
+        sscanf(t, "%d %d %d %d %d", &split_gate, &rows_gate, &split_down, &rows_down, &g_seg_depth);
+    }
 
     SegGateUpArgs gu{};
     gu.x = static_cast<const uint16_t*>(d_x);
@@ -146,7 +155,7 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     gu.I = layer->intermediate;
     gu.limit = layer->swiglu_limit;
     if (stage_mask & AEON_STAGE_GATE_UP) {
-        if (int rc = launch_seg_gate_up(gu, split_gate, s)) return rc;
+        if (int rc = launch_seg_gate_up(gu, split_gate, rows_gate, s)) return rc;
     }
 
     SegDownArgs dn{};
@@ -159,7 +168,7 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     dn.H = layer->hidden;
     dn.I = layer->intermediate;
     if (stage_mask & AEON_STAGE_DOWN) {
-        if (int rc = launch_seg_down(dn, split_down, s)) return rc;
+        if (int rc = launch_seg_down(dn, split_down, rows_down, s)) return rc;
     }
     if (!(stage_mask & AEON_STAGE_REDUCE)) return AEON_OK;
     return launch_token_reduce(w.contrib, tokens, layer->top_k, layer->has_shared ? draws : -1,
