@@ -51,6 +51,12 @@ int launch_seg_down(const SegDownArgs& a, int k_split, int row_tiles, hipStream_
 
 extern int g_seg_depth;
 
+// Prefill form: position tiles of up to kGroupedTokens per expert, weights dequantised into
+// MFMA fragments and reused across the tile's token tiles.
+constexpr int kGroupedTokensPerTile = 128;
+int launch_grouped_gate_up(const SegGateUpArgs& a, hipStream_t stream);
+int launch_grouped_down(const SegDownArgs& a, hipStream_t stream);
+
 // out[t][i] = half( [shared: float(half(contrib[shared_base + t][i]))] +
 //                   sum_{s < slots, ascending} contrib[t*slots + s][i] ),
 // with `initial` (nullable, may alias out) added as the fp16 starting value when there is no

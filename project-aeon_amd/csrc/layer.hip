@@ -12,6 +12,9 @@ extern "C" size_t aeon_router_logits_workspace_bytes(int tokens, int hidden, int
 
 namespace aeon355 {
 
+// Up to this many tokens a step is a decode batch; above it, a prefill chunk.
+constexpr int kDecodeMaxTokens = 64;
+
 static size_t align_up(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
 
 struct LayerWorkspace {
@@ -125,8 +128,12 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     p.seg_first = w.seg_first;
     p.seg_count = w.seg_count;
     p.seg_total = w.seg_total;
-    p.seg_tokens = kSegTokens;
-    p.seg_capacity = w.seg_capacity;
+    // A decode batch walks 16-position segments with the weight-streaming kernels; a prefill
+    // chunk walks 128-position tiles with the grouped GEMM.
+    const bool grouped = tokens > kDecodeMaxTokens;
+    const int lists = layer->experts + (layer->has_shared ? 1 : 0);
+    p.seg_tokens = grouped ? kGroupedTokensPerTile : kSegTokens;
+    p.seg_capacity = grouped ? lists + w.positions / kGroupedTokensPerTile + 1 : w.seg_capacity;
     if (stage_mask & AEON_STAGE_PERMUTATION) {
         if (int rc = launch_permutation(p, s)) return rc;
     }
@@ -149,13 +156,16 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     gu.x_stride = x_stride;
     gu.row_index = w.token_indices;
     gu.experts = layer->d_experts;
-    gu.seg = SegmentList{w.seg_expert, w.seg_first, w.seg_count, w.seg_total, w.seg_capacity};
+    gu.seg = SegmentList{w.seg_expert, w.seg_first, w.seg_count, w.seg_total, p.seg_capacity};
     gu.hidden = w.hidden;
     gu.H = layer->hidden;
     gu.I = layer->intermediate;
     gu.limit = layer->swiglu_limit;
     if (stage_mask & AEON_STAGE_GATE_UP) {
-        if (int rc = launch_seg_gate_up(gu, split_gate, rows_gate, s)) return rc;
+        if (int rc = grouped ? launch_grouped_gate_up(gu, s)
+                             : launch_seg_gate_up(gu, split_gate, rows_gate, s)) {
+            return rc;
+        }
     }
 
     SegDownArgs dn{};
@@ -168,7 +178,10 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     dn.H = layer->hidden;
     dn.I = layer->intermediate;
     if (stage_mask & AEON_STAGE_DOWN) {
-        if (int rc = launch_seg_down(dn, split_down, rows_down, s)) return rc;
+        if (int rc = grouped ? launch_grouped_down(dn, s)
+                             : launch_seg_down(dn, split_down, rows_down, s)) {
+            return rc;
+        }
     }
     if (!(stage_mask & AEON_STAGE_REDUCE)) return AEON_OK;
     return launch_token_reduce(w.contrib, tokens, layer->top_k, layer->has_shared ? draws : -1,

@@ -11,7 +11,11 @@ namespace aeon355 {
 constexpr int kRouterTokenTile = 16;
 constexpr int kRouterMaxExperts = 1024;
 
-// partial[c][t][e] = sum_{h in chunk c, ascending} x[t][h] * Wr[h][e]
+// partial[c][t][e] = sum over the rows h of chunk c of x[t][h] * Wr[h][e].
+// One workgroup = (chunk, tile of 16 tokens), four waves. A wave takes every fourth row of the
+// chunk and reads it as one coalesced float4-per-lane load (64 lanes x 4 experts = 256 experts
+// per pass), eight rows in flight; the four waves' sums meet in LDS in wave order, so the
+// result does not depend on timing.
 __global__ __launch_bounds__(256) void router_logits_partial_kernel(
     const uint16_t* __restrict__ x, long x_stride, const float* __restrict__ wr,
     float* __restrict__ partial, int tokens, int hidden, int experts, int chunk_rows) {
@@ -19,37 +23,89 @@ __global__ __launch_bounds__(256) void router_logits_partial_kernel(
     const int t0 = blockIdx.y * kRouterTokenTile;
     const int h0 = chunk * chunk_rows;
     const int h1 = min(hidden, h0 + chunk_rows);
-    extern __shared__ float xs[];  // [kRouterTokenTile][chunk_rows]
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    extern __shared__ float lds[];
+    float* xs = lds;                                  // [chunk_rows][kRouterTokenTile]
+    float* sums = lds + chunk_rows * kRouterTokenTile;  // [3][kRouterTokenTile][256]: waves 1..3
     for (int i = threadIdx.x; i < kRouterTokenTile * chunk_rows; i += blockDim.x) {
-        const int t = i / chunk_rows;
-        const int h = h0 + i % chunk_rows;
+        const int t = i % kRouterTokenTile;
+        const int h = h0 + i / kRouterTokenTile;
         xs[i] = (t0 + t < tokens && h < h1) ? half_bits_to_float(x[(t0 + t) * x_stride + h]) : 0.0f;
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < experts; e += blockDim.x) {
-        float acc[kRouterTokenTile];
+    for (int e0 = 0; e0 < experts; e0 += 256) {
+        const int e = e0 + lane * 4;
+        float4_t acc[kRouterTokenTile];
 #pragma unroll
-        for (int t = 0; t < kRouterTokenTile; ++t) acc[t] = 0.0f;
-        for (int h = h0; h < h1; ++h) {
-            const float w = wr[static_cast<size_t>(h) * experts + e];
+        for (int t = 0; t < kRouterTokenTile; ++t) acc[t] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        constexpr int kRows = 8;
+        for (int hb = h0 + wave; hb < h1; hb += 4 * kRows) {
+            float4_t w[kRows];
 #pragma unroll
-            for (int t = 0; t < kRouterTokenTile; ++t) acc[t] += xs[t * chunk_rows + (h - h0)] * w;
-        }
+            for (int j = 0; j < kRows; ++j) {
+                const int h = hb + 4 * j;
+                w[j] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                if (h < h1 && e + 3 < experts) {
+                    w[j] = *reinterpret_cast<const float4_t*>(wr + static_cast<size_t>(h) * experts + e);
+                } else if (h < h1) {
+                    for (int q = 0; q < 4; ++q) {
+                        if (e + q < experts) w[j][q] = wr[static_cast<size_t>(h) * experts + e + q];
+                    }
+                }
+            }
 #pragma unroll
-        for (int t = 0; t < kRouterTokenTile; ++t) {
-            if (t0 + t < tokens) {
-                partial[(static_cast<size_t>(chunk) * tokens + t0 + t) * experts + e] = acc[t];
+            for (int j = 0; j < kRows; ++j) {
+                const int h = hb + 4 * j;
+                if (h < h1) {
+                    const float* xrow = xs + (h - h0) * kRouterTokenTile;
+#pragma unroll
+                    for (int t = 0; t < kRouterTokenTile; ++t) acc[t] += xrow[t] * w[j];
+                }
             }
         }
+        if (wave > 0) {
+#pragma unroll
+            for (int t = 0; t < kRouterTokenTile; ++t) {
+                *reinterpret_cast<float4_t*>(sums + ((wave - 1) * kRouterTokenTile + t) * 256 +
+                                             lane * 4) = acc[t];
+            }
+        }
+        __syncthreads();
+        if (wave == 0) {
+#pragma unroll
+            for (int t = 0; t < kRouterTokenTile; ++t) {
+                float4_t v = acc[t];
+#pragma unroll
+                for (int w2 = 0; w2 < 3; ++w2) {
+                    v += *reinterpret_cast<const float4_t*>(sums + (w2 * kRouterTokenTile + t) * 256 +
+                                                            lane * 4);
+                }
+                if (t0 + t < tokens) {
+                    float* dst = partial + (static_cast<size_t>(chunk) * tokens + t0 + t) * experts + e;
+                    for (int q = 0; q < 4; ++q) {
+                        if (e + q < experts) dst[q] = v[q];
+                    }
+                }
+            }
+        }
+        __syncthreads();
     }
 }
 
+// logits[i] = sum over chunks, ascending (eight loads in flight).
 __global__ __launch_bounds__(256) void router_logits_reduce_kernel(
     const float* __restrict__ partial, float* __restrict__ logits, int chunks, size_t count) {
     const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= count) return;
     float acc = 0.0f;
-    for (int c = 0; c < chunks; ++c) acc += partial[static_cast<size_t>(c) * count + i];
+    for (int c0 = 0; c0 < chunks; c0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = c0 + j < chunks ? partial[static_cast<size_t>(c0 + j) * count + i] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc += v[j];
+    }
     logits[i] = acc;
 }
 
@@ -61,12 +117,12 @@ __device__ __forceinline__ double router_score(double logit, int score_kind) {
 
 // One wave per token. Lane l owns experts l, l+64, ...; each of the k rounds is a lane-local
 // scan in ascending index followed by a wave arg-max whose ties go to the lower index.
+template <int kPerLane>
 __global__ __launch_bounds__(64) void router_topk_kernel(
     const float* __restrict__ logits, const float* __restrict__ bias,
     const int64_t* __restrict__ hash_table, const int32_t* __restrict__ token_ids,
     float* __restrict__ topk_weights, int32_t* __restrict__ topk_indices, int experts, int top_k,
     float scaling, int renormalize, int score_kind) {
-    constexpr int kPerLane = kRouterMaxExperts / 64;
     const int token = blockIdx.x;
     const int lane = threadIdx.x;
     const float* row = logits + static_cast<size_t>(token) * experts;
@@ -141,12 +197,15 @@ __global__ __launch_bounds__(64) void router_topk_kernel(
 }
 
 int router_logits_chunks(int tokens, int hidden) {
-    // about 512 workgroups: plenty of chunks for a decode batch, few for a prefill chunk
+    // about 256 workgroups: many short chunks for a decode batch, few for a prefill chunk
     const int tiles = (tokens + kRouterTokenTile - 1) / kRouterTokenTile;
-    int chunks = 512 / (tiles > 0 ? tiles : 1);
+    int chunks = 256 / (tiles > 0 ? tiles : 1);
+    if (chunks > 64) chunks = 64;
     if (chunks < 1) chunks = 1;
     const int max_chunks = (hidden + 31) / 32;
     if (chunks > max_chunks) chunks = max_chunks;
+    const int min_chunks = (hidden + 127) / 128;  // a chunk's activations must fit in LDS
+    if (chunks < min_chunks) chunks = min_chunks;
     return chunks;
 }
 
@@ -175,7 +234,7 @@ extern "C" int aeon_router_logits(const void* d_x, int x_stride, const float* d_
     const int chunks = router_logits_chunks(tokens, hidden);
     const int chunk_rows = (hidden + chunks - 1) / chunks;
     const int tiles = (tokens + kRouterTokenTile - 1) / kRouterTokenTile;
-    const size_t lds = static_cast<size_t>(kRouterTokenTile) * chunk_rows * sizeof(float);
+    const size_t lds = static_cast<size_t>(kRouterTokenTile) * (chunk_rows + 3 * 256) * sizeof(float);
     AEON_REQUIRE(lds <= 64 * 1024, AEON_ERR_INVALID_ARGUMENT,
                  "%s: hidden=%d needs %zu bytes of LDS per chunk", who, hidden, lds);
     hipStream_t s = as_stream(stream);
@@ -208,9 +267,15 @@ extern "C" int aeon_moe_router(const float* d_logits, const float* d_bias,
     AEON_REQUIRE((d_hash_table == nullptr) == (d_token_ids == nullptr), AEON_ERR_INVALID_ARGUMENT,
                  "%s: the hash branch needs both the table and the token ids", who);
     if (tokens == 0) return AEON_OK;
-    router_topk_kernel<<<tokens, 64, 0, as_stream(stream)>>>(
-        d_logits, d_bias, d_hash_table, d_token_ids, d_topk_weights, d_topk_indices, experts, top_k,
-        routed_scaling_factor, renormalize, score_kind);
+    if (experts <= 256) {
+        router_topk_kernel<4><<<tokens, 64, 0, as_stream(stream)>>>(
+            d_logits, d_bias, d_hash_table, d_token_ids, d_topk_weights, d_topk_indices, experts,
+            top_k, routed_scaling_factor, renormalize, score_kind);
+    } else {
+        router_topk_kernel<kRouterMaxExperts / 64><<<tokens, 64, 0, as_stream(stream)>>>(
+            d_logits, d_bias, d_hash_table, d_token_ids, d_topk_weights, d_topk_indices, experts,
+            top_k, routed_scaling_factor, renormalize, score_kind);
+    }
     AEON_LAUNCH_CHECK();
     return AEON_OK;
 }
