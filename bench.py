@@ -42,6 +42,62 @@ def matrix_bytes(n, k):
     return n * k // 2 + n * (k // 128) * 2
 
 
+def run_prefill(layer, moe, capi, synth, torch, np, H, I, E, K_TOP, SEED, steps, warmup):
+    """BASELINE config 3: 2048 tokens, top-8 of 256 experts with Zipf(1.1) popularity, through the
+    permutation -> grouped gate+up GEMM + SwiGLU -> grouped W2 GEMM -> fixed-order reduce path.
+    FLOPs are the algorithmic 2*positions*3*H*I (routed draws + the shared expert's tokens)."""
+    T = 2048
+    ids_h, w_h = synth.zipf_routing(SEED, T, E, K_TOP, s=1.1)
+    counts = np.bincount(ids_h.ravel(), minlength=E)
+    x = torch.from_numpy(synth.activations(SEED, T, H, unit=3)).cuda()
+    ids = torch.from_numpy(ids_h).cuda()
+    w = torch.from_numpy(w_h).cuda()
+    out = torch.empty(T, H, dtype=torch.float16, device="cuda")
+    ws = layer._workspace(T)
+
+    def stages(mask):
+        capi.call("aeon_moe_layer_routed_stages", C.byref(layer.cfg), capi.vp(x), x.stride(0), T,
+                  capi.vp(ids), capi.vp(w), capi.vp(out), out.stride(0), capi.vp(ws),
+                  C.c_size_t(ws.numel()), mask, moe.stream_ptr())
+
+    def timed(mask, reps):
+        stages(mask)
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            stages(mask)
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / reps
+
+    for _ in range(max(warmup, 1)):
+        stages(15)
+    reps = max(3, min(steps, 10))
+    all_ms = timed(15, reps)
+    gu_ms = timed(2, reps)
+    dn_ms = timed(4, reps)
+    routed_flop = 2.0 * T * K_TOP * 3 * H * I
+    shared_flop = 2.0 * T * 3 * H * I
+    tiles = int(np.ceil(counts / 128.0).sum()) + T // 128
+    return {
+        "workload": "config3: prefill 2048 tokens, top-8 of %d experts, Zipf(1.1), + shared" % E,
+        "ms_per_step": round(all_ms, 4),
+        "tokens_per_s": round(T / (all_ms * 1e-3), 1),
+        "routed_tflop": round(routed_flop / 1e12, 4), "shared_tflop": round(shared_flop / 1e12, 4),
+        "tflops": round((routed_flop + shared_flop) / (all_ms * 1e-3) / 1e12, 1),
+        "frac_of_mfma_peak": round((routed_flop + shared_flop) / (all_ms * 1e-3) / 1e12 /
+                                   MFMA_F16_PEAK_TFLOPS, 4),
+        "gate_up_ms": round(gu_ms, 4),
+        "gate_up_tflops": round((routed_flop + shared_flop) * 2 / 3 / (gu_ms * 1e-3) / 1e12, 1),
+        "down_ms": round(dn_ms, 4),
+        "down_tflops": round((routed_flop + shared_flop) / 3 / (dn_ms * 1e-3) / 1e12, 1),
+        "histogram": {"max": int(counts.max()), "empty": int((counts == 0).sum()),
+                      "below_16": int((counts < 16).sum()), "position_tiles": tiles},
+        "weight_bytes_floor": int((int((counts > 0).sum()) + 1) * 3 * matrix_bytes(I, H)),
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -52,6 +108,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
     ap.add_argument("--cpu-tokens", type=int, default=4,
                     help="tokens of the batch the CPU oracle is timed on")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the config-3 prefill leg")
     ap.add_argument("--sweep", action="store_true",
                     help="also report batch 1/8/32/64 in the `sweep` field")
     args = ap.parse_args()
@@ -161,6 +218,11 @@ def main():
             sweep.append({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()
                           if k not in ("x", "ids", "w", "out")})
 
+    prefill = None
+    if not args.no_prefill:
+        prefill = run_prefill(layer, moe, capi, synth, torch, np, H, I, E, K_TOP, SEED, args.steps,
+                              args.warmup)
+
     cpu = None
     if not args.no_cpu:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
@@ -231,6 +293,8 @@ def main():
         "cpu_baseline": cpu,
         "setup_s": round(setup_s, 1),
     }
+    if prefill is not None:
+        result["prefill"] = prefill
     if sweep is not None:
         result["sweep"] = sweep
     print(json.dumps(result))

@@ -259,6 +259,36 @@ int aeon_moe_layer_decode(const aeon_moe_layer* layer, const void* d_x, int x_st
 const float* aeon_moe_layer_logits(const aeon_moe_layer* layer, int tokens, void* d_workspace);
 
 /* ------------------------------------------------------------------------------------------
+ * Hyper-connection stream mix (hc_mult = 4)
+ * ---------------------------------------------------------------------------------------- */
+
+/* hc_sinkhorn_normalize_kernel launch, src/architecture/deepseek_v4/kernels/
+ * hc_sinkhorn.hpp:151-255: mixes [tokens][24] -> pre [tokens][4] = sigmoid(m*s0+b)+pre_eps,
+ * post [tokens][4] = sigmoid(m*s1+b)*post_alpha, comb [tokens][16] (comb[i*4+j], i the
+ * contraction stream, j the output stream): row softmax + eps, column normalisation, then
+ * (iters-1) x (row, column), every denominator + sinkhorn_eps. */
+int aeon_hc_sinkhorn_normalize(const float* d_mixes, const float* d_hc_scale,
+                               const float* d_hc_base, float* d_pre_mix, float* d_post_mix,
+                               float* d_comb_mix, int tokens, float hc_pre_eps,
+                               float hc_sinkhorn_eps, float hc_post_alpha, int sinkhorn_iters,
+                               void* stream);
+/* hc_pre_combine_kernel launch, hc_sinkhorn.hpp:94-147: layer_input[t][h] =
+ * sum_j pre[j]*residual[t][j][h] -> fp16. The residual is fp32 (the reference's) or fp16, element
+ * (t, j, h) at t*token_stride + j*stream_stride + h; pre_token_stride 4 = per-token mixes,
+ * 0 = one mix for every token. */
+int aeon_hc_pre_combine(const void* d_residual, int residual_is_f32, long token_stride,
+                        long stream_stride, const float* d_pre_mix, int pre_token_stride,
+                        void* d_layer_input, long out_stride, int tokens, int hidden,
+                        void* stream);
+/* hc_post_kernel launch, hc_sinkhorn.hpp:259-290: out[t][j][h] = post[j]*layer_out[t][h] +
+ * sum_i comb[i*4+j]*residual_in[t][i][h], fp16 streams, fp32 math. mix_per_token 1 = post/comb
+ * per token, 0 = shared by all tokens. Input and output residuals must not alias. */
+int aeon_hc_post(const void* d_layer_out, long layer_out_stride, const void* d_residual_in,
+                 long token_stride, long stream_stride, const float* d_post_mix,
+                 const float* d_comb_mix, int mix_per_token, void* d_residual_out, int tokens,
+                 int hidden, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Synthetic experts on the device (benchmarks and tests)
  * ---------------------------------------------------------------------------------------- */
 

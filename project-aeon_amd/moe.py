@@ -151,3 +151,65 @@ class MoeLayer:
                   capi.vp(out), tokens, self.cfg.hidden, E, capi.vp(ws), C.c_size_t(ws.numel()),
                   stream_ptr())
         return out
+
+
+class HyperConnection:
+    """The static 4-stream mix of one layer boundary: mixes [24] -> (pre [4], post [4], comb [16])
+    by the Sinkhorn kernel (20 iterations), shared by every token."""
+
+    def __init__(self, mixes, hc_scale=(1.0, 1.0, 1.0), hc_base=None, pre_eps=1e-6,
+                 sinkhorn_eps=1e-6, post_alpha=2.0, iters=20, device="cuda"):
+        self.mixes = torch.as_tensor(np.asarray(mixes, dtype=np.float32)).reshape(1, 24).to(device)
+        self.scale = torch.as_tensor(np.asarray(hc_scale, dtype=np.float32)).to(device)
+        base = np.zeros(24, dtype=np.float32) if hc_base is None else np.asarray(hc_base, np.float32)
+        self.base = torch.as_tensor(base).to(device)
+        self.pre = torch.empty(1, 4, dtype=torch.float32, device=device)
+        self.post = torch.empty(1, 4, dtype=torch.float32, device=device)
+        self.comb = torch.empty(1, 16, dtype=torch.float32, device=device)
+        capi.call("aeon_hc_sinkhorn_normalize", capi.vp(self.mixes), capi.vp(self.scale),
+                  capi.vp(self.base), capi.vp(self.pre), capi.vp(self.post), capi.vp(self.comb), 1,
+                  C.c_float(pre_eps), C.c_float(sinkhorn_eps), C.c_float(post_alpha), iters,
+                  stream_ptr())
+
+    def pre_combine(self, residual, out):
+        """residual fp16 [4][tokens][hidden] -> out fp16 [tokens][hidden]."""
+        streams, tokens, hidden = residual.shape
+        capi.call("aeon_hc_pre_combine", capi.vp(residual), 0, C.c_long(residual.stride(1)),
+                  C.c_long(residual.stride(0)), capi.vp(self.pre), 0, capi.vp(out),
+                  C.c_long(out.stride(0)), tokens, hidden, stream_ptr())
+        return out
+
+    def post_mix(self, layer_out, residual_in, residual_out):
+        streams, tokens, hidden = residual_in.shape
+        capi.call("aeon_hc_post", capi.vp(layer_out), C.c_long(layer_out.stride(0)),
+                  capi.vp(residual_in), C.c_long(residual_in.stride(1)),
+                  C.c_long(residual_in.stride(0)), capi.vp(self.post), capi.vp(self.comb), 0,
+                  capi.vp(residual_out), tokens, hidden, stream_ptr())
+        return residual_out
+
+
+class LayerStack:
+    """BASELINE config 4: stacked MoE layers with the hyper-connection residual mix between them.
+    Per layer: x = pre-combine(residual); y = MoE(x); residual = post-mix(y, residual)."""
+
+    def __init__(self, layers, mixes):
+        assert len(layers) == len(mixes)
+        self.layers = layers
+        self.mixes = mixes
+
+    def step(self, residual, scratch=None, trace=None):
+        """residual fp16 [4][tokens][hidden]; returns the new residual (a different buffer)."""
+        streams, tokens, hidden = residual.shape
+        if scratch is None:
+            scratch = (torch.empty_like(residual), torch.empty(tokens, hidden, dtype=torch.float16,
+                                                               device=residual.device))
+        other, x = scratch
+        for layer, hc in zip(self.layers, self.mixes):
+            hc.pre_combine(residual, x)
+            y, ids, w = layer.decode(x)
+            hc.post_mix(y, residual, other)
+            if trace is not None:
+                trace.append((residual.clone(), x.clone(), ids.clone(), w.clone(), y.clone(),
+                              other.clone()))
+            residual, other = other, residual
+        return residual

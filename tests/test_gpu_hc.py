@@ -1,0 +1,141 @@
+"""GPU parity for the hyper-connection kernels and the stacked-layer decode step (config 4)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _setup():
+    import torch
+    assert torch.cuda.is_available()
+    import helpers
+    from project_aeon_amd import capi, moe, synth
+    return torch, helpers, capi, moe, synth
+
+
+def test_sinkhorn_against_oracle_and_closed_forms(orc):
+    torch, h, capi, moe, synth = _setup()
+    rng = np.random.default_rng(3)
+    T = 33
+    mixes = rng.normal(size=(T, 24)).astype(np.float32)
+    mixes[0] = 0.0
+    scale = rng.normal(size=3).astype(np.float32)
+    base = rng.normal(size=24).astype(np.float32)
+    base0 = np.zeros(24, dtype=np.float32)
+    for iters, b in ((20, base), (1, base), (20, base0)):
+        d_m, d_s, d_b = h.to_dev(mixes), h.to_dev(scale), h.to_dev(b)
+        pre = torch.zeros(T, 4, device="cuda")
+        post = torch.zeros(T, 4, device="cuda")
+        comb = torch.zeros(T, 16, device="cuda")
+        capi.call("aeon_hc_sinkhorn_normalize", capi.vp(d_m), capi.vp(d_s), capi.vp(d_b),
+                  capi.vp(pre), capi.vp(post), capi.vp(comb), T, C.c_float(1e-6), C.c_float(1e-6),
+                  C.c_float(2.0), iters, h.stream_ptr())
+        pre, post, comb = pre.cpu().numpy(), post.cpu().numpy(), comb.cpu().numpy()
+        for t in range(T):
+            op, oq, oc = orc.hc_sinkhorn(mixes[t], scale, b, 4, orc.hc_params(sinkhorn_iters=iters))
+            assert np.abs(pre[t] - op).max() <= 1e-5      # tests/test_hc_sinkhorn.cpp tolerances
+            assert np.abs(post[t] - oq).max() <= 1e-5
+            assert np.abs(comb[t] - oc).max() <= 1e-5
+        if iters == 20:
+            c = comb.reshape(T, 4, 4)
+            # doubly stochastic up to the eps the fixed point carries (row/col sums 1 - eps)
+            assert np.abs(c.sum(1) - 1).max() < 1e-4 and np.abs(c.sum(2) - 1).max() < 1e-4
+        if b is base0:
+            # zero logits: every entry 1/4, off by the eps share (tests/test_v4_hc_oracle.cpp:371-404)
+            assert np.abs(comb[0] - 0.25).max() < 1e-6
+            assert np.abs(pre[0] - (0.5 + 1e-6)).max() < 1e-6 and np.abs(post[0] - 1.0).max() < 1e-6
+
+
+def test_pre_combine_and_post_against_oracle(orc):
+    torch, h, capi, moe, synth = _setup()
+    rng = np.random.default_rng(4)
+    T, H = 5, 1024
+    res = rng.normal(size=(4, T, H)).astype(np.float16)     # stream-major, as config 4 lays it out
+    lo = rng.normal(size=(T, H)).astype(np.float16)
+    mixes = rng.normal(size=24).astype(np.float32)
+    hc = moe.HyperConnection(mixes)
+    pre, post, comb = orc.hc_sinkhorn(mixes, np.ones(3), np.zeros(24), 4)
+    assert np.abs(hc.pre.cpu().numpy()[0] - pre).max() <= 1e-5
+    d_res, d_lo = h.dev_half(res), h.dev_half(lo)
+    x = torch.zeros(T, H, dtype=torch.float16, device="cuda")
+    hc.pre_combine(d_res, x)
+    out = torch.zeros_like(d_res)
+    hc.post_mix(d_lo, d_res, out)
+    x, out = x.cpu().numpy().astype(np.float64), out.cpu().numpy().astype(np.float64)
+    dpre = hc.pre.cpu().numpy()[0].astype(np.float64)
+    dpost = hc.post.cpu().numpy()[0].astype(np.float64)
+    dcomb = hc.comb.cpu().numpy()[0].astype(np.float64)
+    for t in range(T):
+        r = res[:, t, :].astype(np.float64)
+        want_x = orc.hc_pre_combine(r, dpre, H)
+        assert np.abs(x[t] - want_x).max() <= 1e-4 + 1e-3 * np.abs(want_x).max()
+        want = orc.hc_post(lo[t].astype(np.float64), r, dpost, dcomb, H)
+        assert np.abs(out[:, t, :] - want).max() <= 1e-4 + 1e-3 * np.abs(want).max()
+        # the transposed reading of comb is a different function, and the kernel is not on it
+        wrong = orc.hc_post(lo[t].astype(np.float64), r, dpost, dcomb, H, transpose_comb=True)
+        assert np.abs(wrong - want).max() > 1e-2
+        assert np.abs(out[:, t, :] - wrong).max() > 1e-2
+    # fp32 residual form of the pre-combine (the reference kernel's input type), per-token mixes
+    res32 = rng.normal(size=(T, 4, H)).astype(np.float32)
+    pre_t = rng.random((T, 4)).astype(np.float32)
+    x2 = torch.zeros(T, H, dtype=torch.float16, device="cuda")
+    d_res32, d_pre = h.to_dev(res32), h.to_dev(pre_t)
+    capi.call("aeon_hc_pre_combine", capi.vp(d_res32), 1, C.c_long(4 * H), C.c_long(H),
+              capi.vp(d_pre), 4, capi.vp(x2), C.c_long(H), T, H, h.stream_ptr())
+    want2 = np.einsum("tj,tjh->th", pre_t.astype(np.float64), res32.astype(np.float64))
+    assert np.abs(x2.cpu().numpy() - want2).max() <= 1e-4 + 1e-3 * np.abs(want2).max()
+    with pytest.raises(ValueError):
+        hc.post_mix(d_lo, d_res, d_res)
+
+
+@pytest.mark.parametrize("B,H,I,E", [(64, 1024, 512, 16), (4, 7168, 2048, 12)])
+def test_config4_stacked_layers(orc, B, H, I, E):
+    """Four MoE layers with independent seeded weights and the HC mix between them. Each layer is
+    checked against the oracle on the device's own input to that layer and the device's routed
+    ids (the way a composed gate isolates one stage from the rounding of the ones before it)."""
+    torch, h, capi, moe, synth = _setup()
+    k, limit, L = 8, 7.0, 4
+    layers, mixes, host = [], [], []
+    for l in range(L):
+        pool = moe.ExpertPool(E + 1, H, I)
+        assert pool.fill_synthetic(seed=11, first_expert_id=1000 * l) == 0
+        wr, bias = synth.router_weight(11, H, E, unit=l), synth.router_bias(11, E, unit=l)
+        d_wr, d_bias = h.to_dev(wr), h.to_dev(bias)
+        layers.append(moe.MoeLayer(pool, E, k, True, limit, d_wr, d_bias, score_kind=1))
+        mix = synth.normal(synth.stream_key(11, synth.STREAM_HC, l), 24).astype(np.float32)
+        mixes.append(moe.HyperConnection(mix))
+        host.append((wr, bias, mix))
+    stack = moe.LayerStack(layers, mixes)
+    res0 = synth.activations(11, 4 * B, H).reshape(4, B, H)
+    trace = []
+    final = stack.step(h.dev_half(res0), trace=trace)
+    torch.cuda.synchronize()
+    assert np.isfinite(final.cpu().numpy()).all()
+    import test_gpu_layer as tl
+    for l, (res_in, x, ids, w, y, res_out) in enumerate(trace):
+        wr, bias, mix = host[l]
+        res_in, x, y = res_in.cpu().numpy(), x.cpu().numpy(), y.cpu().numpy()
+        ids, w, res_out = ids.cpu().numpy(), w.cpu().numpy(), res_out.cpu().numpy()
+        pre, post, comb = orc.hc_sinkhorn(mix, np.ones(3), np.zeros(24), 4)
+        check = range(B) if H <= 1024 else range(min(B, 2))
+        experts = {int(e): h.Expert(11, 1000 * l + int(e), H, I) for t in check for e in ids[t]}
+        shared = h.Expert(11, 1000 * l + E, H, I)
+        for t in check:
+            r = res_in[:, t, :].astype(np.float64)
+            want_x = orc.hc_pre_combine(r, pre, H)
+            assert np.abs(x[t] - want_x).max() <= 2e-3 * np.abs(want_x).max()
+            logits = x[t].astype(np.float64) @ wr.astype(np.float64)
+            oi, ow = orc.router_topk(logits, bias.astype(np.float64), k, 1.0, 1)
+            assert set(oi) == set(ids[t]) or np.sort(logits)[-9] > np.sort(logits)[-8] - 1e-4
+        rows = list(check)
+        want_y = tl._oracle_layer(orc, h, experts, x[rows], ids[rows], w[rows], shared, limit)
+        assert np.abs(y[rows] - want_y).max() <= 6e-3 * np.abs(want_y).max()
+        for t in check:
+            want_r = orc.hc_post(y[t].astype(np.float64), res_in[:, t, :].astype(np.float64), post,
+                                 comb, H)
+            assert np.abs(res_out[:, t, :] - want_r).max() <= 2e-3 * np.abs(want_r).max()
+    # the step is bit-reproducible
+    again = stack.step(h.dev_half(res0))
+    assert torch.equal(again, final)
