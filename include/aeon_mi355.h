@@ -121,6 +121,25 @@ int aeon_moe_accumulate_fixed_order(const float* d_contrib, int expert_count,
 int aeon_swiglu_clamp(const void* d_gate, const void* d_up, void* d_out, int total_elements,
                       float limit, void* stream);
 
+/* dispatch_aeon_moe_grouped_w13_swiglu_wmma<WAVES,RPW,LPR,MTILES>, src/architecture/deepseek_v4/
+ * kernels/moe_grouped_dispatch.hpp:45-64 (kernel: src/platform/rdna3/moe_grouped_ffn.hpp:75-188,
+ * feed: swizzled_w4a16_feed.hpp:51-140): per expert e of the 8-slot table, over positions
+ * expert_offsets[e]..[e+1): expert_hidden[(e*expert_hidden_tokens + m)*N + n] =
+ * half(clamped_swiglu(W1_e x, W3_e x)) with x = activation row token_indices[position], row
+ * pitch activation_stride (0 = K). Weights dequantised to fp16 with one rounding per weight. */
+int aeon_moe_grouped_w13_swiglu(const void* d_activation, const int* d_expert_offsets,
+                                const int* d_token_indices, const aeon_w13_table* weights,
+                                void* d_expert_hidden, int expert_count, int expert_hidden_tokens,
+                                int N, int K, int rpw, int lpr, float swiglu_limit,
+                                int activation_stride, void* stream);
+/* dispatch_aeon_moe_grouped_w2_wmma, moe_grouped_dispatch.hpp:66-88 (kernel
+ * moe_grouped_ffn.hpp:197-288): contrib[draw_indices[p]*N + n] = draw_weights[p] *
+ * (W2_e . expert_hidden[e][m])[n], one writer per element. */
+int aeon_moe_grouped_w2(const void* d_expert_hidden, const int* d_expert_offsets,
+                        const int* d_draw_indices, const float* d_draw_weights,
+                        const aeon_w2_table* weights, float* d_contrib, int expert_count,
+                        int expert_hidden_tokens, int N, int K, int rpw, int lpr, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Decode kernels over the wave64 packing (the MI355X-native path)
  * ---------------------------------------------------------------------------------------- */

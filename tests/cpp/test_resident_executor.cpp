@@ -1,0 +1,187 @@
+// Gate: the resident-expert executor behind the V4RoutedExpertExecutor seam against a
+// direct-payload executor (the per-token GEMV trio over the `.aeon` payloads, the construction
+// the reference's tests/test_v4_expert_executor.cpp:275-353 uses as its control), on synthetic
+// experts, two layers, six tokens: agreement within a rounding band, a wrong-expert probe that
+// must differ, the chunk form equal to the per-token form, and the protocol errors.
+#include "architecture/deepseek_v4/kernels/moe_gemv_dispatch.hpp"
+#include "architecture/deepseek_v4/moe/v4_resident_expert_executor.hpp"
+#include "backend/swizzled_w4a16/core/swizzled_expert_format.hpp"
+#include "common.hpp"
+#include "platform/ops/moe_accumulate.hpp"
+#include "test_device.hpp"
+
+namespace kernel = aeon::kernel;
+namespace core = aeon::core;
+
+constexpr int kHidden = 4096, kIntermediate = 2048, kSlots = 6, kExperts = 12, kLayers = 2, kTokens = 6;
+constexpr float kLimit = 10.0f;
+constexpr core::SwizzledExpertLayout kL = core::swizzled_expert_layout(kHidden, kIntermediate);
+
+struct DeviceExpert {
+    uint8_t* payload;  // `.aeon` layout, group-32 scales replicated from group-128
+    void* a64[6];      // wave64 packing
+};
+
+static DeviceExpert make_expert(int id) {
+    DeviceExpert e{};
+    GATE_HIP(hipMalloc(&e.payload, kL.bytes));
+    const size_t off[3][2] = {{kL.w1_packed, kL.w1_scale}, {kL.w3_packed, kL.w3_scale}, {kL.w2_packed, kL.w2_scale}};
+    const int shape[3][4] = {{kIntermediate, kHidden, 4, 8}, {kIntermediate, kHidden, 4, 8}, {kHidden, kIntermediate, 8, 4}};
+    for (int m = 0; m < 3; ++m) {
+        aeon355::throw_on_error(aeon_synth_matrix_swizzled(77, id, m, shape[m][0], shape[m][1], shape[m][2],
+                                                           shape[m][3], e.payload + off[m][0],
+                                                           e.payload + off[m][1], nullptr));
+        GATE_HIP(hipMalloc(&e.a64[2 * m], aeon_a64_packed_bytes(shape[m][0], shape[m][1])));
+        GATE_HIP(hipMalloc(&e.a64[2 * m + 1], aeon_a64_scale_bytes(shape[m][0], shape[m][1])));
+        aeon355::throw_on_error(aeon_a64_repack_device(e.payload + off[m][0], e.payload + off[m][1],
+                                                       shape[m][0], shape[m][1], shape[m][2], shape[m][3],
+                                                       e.a64[2 * m], e.a64[2 * m + 1], nullptr, nullptr));
+    }
+    return e;
+}
+
+// The control: payloads handed straight to the fused dispatches, no pool, no table.
+class DirectPayloadExecutor final : public core::V4RoutedExpertExecutor {
+public:
+    explicit DirectPayloadExecutor(const std::vector<std::vector<DeviceExpert>>& experts) : experts_(experts) {
+        GATE_HIP(hipMalloc(&hidden_, sizeof(half) * kernel::kAeonSwizzledMaxExperts * kIntermediate));
+        GATE_HIP(hipMalloc(&contrib_, sizeof(float) * kSlots * kHidden));
+    }
+    int wrong_slot{-1};
+    int wrong_expert{0};
+    void on_routing_ready(uint32_t, uint32_t, const std::vector<int32_t>& ids, const std::vector<float>&) override {
+        ids_ = ids;
+    }
+    void accumulate_routed(uint32_t layer, uint32_t, const half* x, const float* w, half* accum) override {
+        kernel::SwizzledW13ExpertPtrs w13{};
+        kernel::SwizzledW2ExpertPtrs w2{};
+        for (int k = 0; k < kSlots; ++k) {
+            const uint8_t* base = experts_[layer][k == wrong_slot ? wrong_expert : ids_[k]].payload;
+            w13.w1[k] = reinterpret_cast<const uint4*>(base + kL.w1_packed);
+            w13.s1[k] = reinterpret_cast<const half*>(base + kL.w1_scale);
+            w13.w3[k] = reinterpret_cast<const uint4*>(base + kL.w3_packed);
+            w13.s3[k] = reinterpret_cast<const half*>(base + kL.w3_scale);
+            w2.w2[k] = reinterpret_cast<const uint4*>(base + kL.w2_packed);
+            w2.s2[k] = reinterpret_cast<const half*>(base + kL.w2_scale);
+        }
+        kernel::dispatch_dsv4_moe_gemv_w13_swiglu<8, 4, 8, 16>(x, w13, hidden_, nullptr, kHidden, kSlots,
+                                                               kIntermediate, kHidden, kLimit);
+        kernel::dispatch_aeon_moe_fused_w2_contrib<8, 8, 4, 16>(hidden_, w2, w, contrib_, kSlots, kHidden,
+                                                                kIntermediate);
+        kernel::moe_accumulate_fixed_order_kernel<<<(kHidden + 255) / 256, 256>>>(contrib_, kSlots, accum,
+                                                                                  accum, kHidden);
+    }
+
+private:
+    const std::vector<std::vector<DeviceExpert>>& experts_;
+    std::vector<int32_t> ids_;
+    half* hidden_{nullptr};
+    float* contrib_{nullptr};
+};
+
+static double max_abs_over_peak(const std::vector<half>& a, const std::vector<half>& b, double* peak_out) {
+    double max_abs = 0, peak = 0;
+    for (size_t i = 0; i < a.size(); ++i) {
+        max_abs = std::fmax(max_abs, std::fabs(__half2float(a[i]) - __half2float(b[i])));
+        peak = std::fmax(peak, std::fabs(__half2float(a[i])));
+    }
+    if (peak_out) *peak_out = peak;
+    return max_abs / std::fmax(peak, 1e-30);
+}
+
+int main() {
+    aeon::test::select_test_device(true);
+    std::vector<std::vector<DeviceExpert>> experts(kLayers);
+    std::vector<aeon_a64_expert*> d_tables(kLayers);
+    std::vector<aeon_moe_layer> layers(kLayers);
+    for (int l = 0; l < kLayers; ++l) {
+        std::vector<aeon_a64_expert> table(kExperts);
+        for (int e = 0; e < kExperts; ++e) {
+            experts[l].push_back(make_expert(100 * l + e));
+            const DeviceExpert& d = experts[l].back();
+            table[e] = aeon_a64_expert{d.a64[0], d.a64[1], d.a64[2], d.a64[3], d.a64[4], d.a64[5]};
+        }
+        d_tables[l] = to_device(table);
+        layers[l] = aeon_moe_layer{kHidden, kIntermediate, kExperts, kSlots, 0, kLimit, AEON_ROUTER_SCORE_SIGMOID,
+                                   1.0f, 1, nullptr, nullptr, d_tables[l]};
+    }
+    GATE_HIP(hipDeviceSynchronize());
+
+    SplitMix rng{0x0E7E1217ull};
+    std::vector<half> x(static_cast<size_t>(kTokens) * kHidden), shared(static_cast<size_t>(kTokens) * kHidden);
+    for (half& v : x) v = __float2half(static_cast<float>(rng.uniform() - 0.5));
+    for (half& v : shared) v = __float2half(static_cast<float>(rng.uniform() - 0.5));
+    half* d_x = to_device(x);
+    core::V4ResidentExpertExecutor resident(layers, 16, nullptr);
+    DirectPayloadExecutor direct(experts);
+
+    double worst = 0, peak = 0, probe = 0, batch_delta = 0;
+    for (int l = 0; l < kLayers; ++l) {
+        std::vector<std::vector<int32_t>> ids(kTokens);
+        std::vector<std::vector<float>> weights(kTokens);
+        std::vector<int32_t> flat_ids;
+        std::vector<float> flat_w;
+        for (int t = 0; t < kTokens; ++t)
+            for (int k = 0; k < kSlots; ++k) {
+                ids[t].push_back((3 * t + 5 * k + l) % kExperts);
+                weights[t].push_back(0.6f / static_cast<float>(k + 1) + 0.02f);
+                flat_ids.push_back(ids[t].back());
+                flat_w.push_back(weights[t].back());
+            }
+        int* d_ids = to_device(flat_ids);
+        float* d_w = to_device(flat_w);
+        half* d_out_res = to_device(shared);
+        half* d_out_dir = to_device(shared);
+        half* d_out_probe = to_device(shared);
+        half* d_out_batch = to_device(shared);
+        for (int t = 0; t < kTokens; ++t) {
+            resident.on_routing_ready(l, 40 + t, ids[t], weights[t]);
+            resident.accumulate_routed(l, 40 + t, d_x + static_cast<size_t>(t) * kHidden, d_w + t * kSlots,
+                                       d_out_res + static_cast<size_t>(t) * kHidden);
+            resident.on_routed_consumed(l, 40 + t);
+            direct.wrong_slot = -1;
+            direct.on_routing_ready(l, 40 + t, ids[t], weights[t]);
+            direct.accumulate_routed(l, 40 + t, d_x + static_cast<size_t>(t) * kHidden, d_w + t * kSlots,
+                                     d_out_dir + static_cast<size_t>(t) * kHidden);
+            direct.wrong_slot = 2;
+            direct.wrong_expert = (ids[t][2] + 1) % kExperts;
+            direct.accumulate_routed(l, 40 + t, d_x + static_cast<size_t>(t) * kHidden, d_w + t * kSlots,
+                                     d_out_probe + static_cast<size_t>(t) * kHidden);
+        }
+        resident.on_routing_ready_batch(l, 100, ids, weights);
+        resident.accumulate_routed_batch(l, 100, kTokens, d_x, kHidden, d_ids, kSlots, d_w, kSlots, d_out_batch,
+                                         kHidden);
+        GATE_HIP(hipGetLastError());
+        GATE_HIP(hipDeviceSynchronize());
+        const size_t n = static_cast<size_t>(kTokens) * kHidden;
+        const std::vector<half> r = to_host(d_out_res, n), d = to_host(d_out_dir, n);
+        double p = 0;
+        worst = std::fmax(worst, max_abs_over_peak(d, r, &p));
+        peak = std::fmax(peak, p);
+        probe = std::fmax(probe, max_abs_over_peak(d, to_host(d_out_probe, n), nullptr));
+        batch_delta = std::fmax(batch_delta, max_abs_over_peak(r, to_host(d_out_batch, n), nullptr));
+    }
+    std::printf("  resident vs direct payload: %.3e of peak %.3e; wrong-expert probe %.3e; chunk vs per-token %.3e\n",
+                worst, peak, probe, batch_delta);
+    expect(peak > 1.0, "signal present");
+    expect(worst <= 2e-3, "resident executor within 2e-3 of peak of the direct-payload control");
+    expect(probe > 50 * worst && probe > 1e-2, "a wrong expert in one slot changes the result materially");
+    expect(batch_delta == 0.0, "chunk form bit-identical to the per-token form");
+
+    bool logic = false, range = false, shape = false;
+    try {
+        resident.accumulate_routed(1, 7, d_x, nullptr, nullptr);  // layer 1 announced positions 100..105
+    } catch (const std::logic_error&) { logic = true; }
+    try {
+        resident.on_routing_ready(1, 7, std::vector<int32_t>(kSlots, 0), std::vector<float>(kSlots, 1.0f));
+        resident.accumulate_routed(1, 9, d_x, nullptr, nullptr);
+    } catch (const std::out_of_range&) { range = true; }
+    try {
+        resident.on_routing_ready(0, 0, std::vector<int32_t>(kSlots - 1, 0), std::vector<float>(kSlots - 1, 1.0f));
+    } catch (const std::invalid_argument&) { shape = true; }
+    expect(logic, "consume before the announced position throws std::logic_error");
+    expect(range, "token index past the batch throws std::out_of_range");
+    expect(shape, "ids not [token, top_k] throws std::invalid_argument");
+    std::printf(g_failures == 0 ? "[PASS] resident executor\n" : "[FAIL] resident executor\n");
+    return g_failures == 0 ? 0 : 1;
+}
