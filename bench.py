@@ -42,6 +42,18 @@ def matrix_bytes(n, k):
     return n * k // 2 + n * (k // 128) * 2
 
 
+def measured_traffic(batch, experts):
+    """HBM bytes per launch of the gate/up kernel from the committed rocprofv3 --pmc runs
+    (FETCH_SIZE, WRITE_SIZE in KiB per dispatch, each scaled by what the same counter reads for a
+    plain copy of known size), or None for a workload that was not profiled."""
+    path = os.path.join(ROOT, "profiles", "traffic_config2_decode_b%d.json" % batch)
+    if experts != 256 or not os.path.exists(path):
+        return None
+    t = json.load(open(path))
+    return int(1024 * (t["fetch_size_kib_per_dispatch"] * t["fetch_scale"] +
+                       t["write_size_kib_per_dispatch"] * t["write_scale"]))
+
+
 def run_prefill(layer, moe, capi, synth, torch, np, H, I, E, K_TOP, SEED, steps, warmup):
     """BASELINE config 3: 2048 tokens, top-8 of 256 experts with Zipf(1.1) popularity, through the
     permutation -> grouped gate+up GEMM + SwiGLU -> grouped W2 GEMM -> fixed-order reduce path.
@@ -286,7 +298,7 @@ def main():
                      "frac": round(main_run["gate_up_gbps"] / HBM_PEAK_GBPS, 4),
                      "avg_launch_ms": round(main_run["gate_up_ms"], 4),
                      "algorithmic_bytes": int(main_run["gate_up_bytes"]),
-                     "traffic": None},
+                     "traffic": measured_traffic(B, E)},
         "down_kernel": {"achieved_gbps": round(main_run["down_gbps"], 1),
                         "avg_launch_ms": round(main_run["down_ms"], 4),
                         "algorithmic_bytes": int(main_run["down_bytes"])},
