@@ -32,7 +32,8 @@ __device__ __forceinline__ half8_t scaled_fragment(uint32_t word, half2_t scale2
 }
 
 template <bool GATE_UP, int R>
-__global__ __launch_bounds__(256) void a64_grouped_kernel(SegGateUpArgs gu, SegDownArgs dn) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void a64_grouped_kernel(
+    SegGateUpArgs gu, SegDownArgs dn) {
     constexpr int NM = GATE_UP ? 2 : 1;
     constexpr int MT = kGroupedMT;
     const SegmentList& seg = GATE_UP ? gu.seg : dn.seg;
@@ -64,25 +65,26 @@ __global__ __launch_bounds__(256) void a64_grouped_kernel(SegGateUpArgs gu, SegD
     // B operand is one conflict-free ds_read_b128 per lane.
     __shared__ half8_t xs[2][MT][4][64];
 
-    // Staging assignment: the tile is MT*16 rows x 256 bytes = 16 pieces of 16 bytes per row;
-    // thread i handles pieces i, i+256, ... (consecutive threads read consecutive 16 bytes).
-    constexpr int kPieces = MT * 16 * 16 / 256;  // per thread
-    const AEON_GLOBAL uint16_t* piece_src[kPieces];
-    int piece_dst[kPieces];
+    // Staging assignment: the tile is MT*4 fragments of 1 KiB (token tile mt, MFMA step st); wave
+    // w stages fragments w*kFrags .. +kFrags-1. Lane (n, chunk) of a fragment fetches 16 bytes of
+    // row mt*16+n at column st*32 + chunk*8 and stores them at the lane's own 16-byte slot, so
+    // the LDS write of a wave is one contiguous KiB (no bank conflicts) and is the exact image
+    // the B-operand read wants.
+    constexpr int kFrags = MT * 4 / 4;  // per wave
+    const AEON_GLOBAL uint16_t* frag_src[kFrags];
 #pragma unroll
-    for (int j = 0; j < kPieces; ++j) {
-        const int idx = threadIdx.x + j * 256;
-        const int row = idx >> 4;         // position within the tile
-        const int piece = idx & 15;       // step = piece / 4, chunk = piece % 4
+    for (int j = 0; j < kFrags; ++j) {
+        const int f = wave * kFrags + j;
+        const int row = (f >> 2) * 16 + n;
         const int live_row = row < count ? row : count - 1;
         const int position = first + live_row;
+        const int column = (f & 3) * 32 + chunk * 8;
         if (GATE_UP) {
             const long src_row = gu.row_index != nullptr ? gu.row_index[position] : position;
-            piece_src[j] = as_global<uint16_t>(gu.x) + src_row * gu.x_stride + piece * 8;
+            frag_src[j] = as_global<uint16_t>(gu.x) + src_row * gu.x_stride + column;
         } else {
-            piece_src[j] = as_global<uint16_t>(dn.hidden) + static_cast<size_t>(position) * dn.I + piece * 8;
+            frag_src[j] = as_global<uint16_t>(dn.hidden) + static_cast<size_t>(position) * dn.I + column;
         }
-        piece_dst[j] = (((row >> 4) * 4 + (piece >> 2)) * 64) + (piece & 3) * 16 + (row & 15);
     }
     half8_t* xs_flat = &xs[0][0][0][0];
     constexpr int kBufferStride = MT * 4 * 64;
@@ -108,23 +110,26 @@ __global__ __launch_bounds__(256) void a64_grouped_kernel(SegGateUpArgs gu, SegD
             }
     };
 
-    half8_t stage[kPieces];
-    auto fetch_tile = [&](int g) {
+    // Activation fragments go from global memory straight into LDS (global_load_lds, 16 bytes
+    // per lane landing at the lane's own slot of the fragment): no staging registers, no LDS
+    // write instructions. The tile for group g+1 is requested at the top of step g into the
+    // other buffer; every wave drains its own requests before the barrier that ends the step.
+    auto fetch_tile = [&](int g, int buffer) {
 #pragma unroll
-        for (int j = 0; j < kPieces; ++j) {
-            stage[j] = *reinterpret_cast<const AEON_GLOBAL half8_t*>(piece_src[j] + g * 128);
-        }
-    };
-    auto publish_tile = [&](int buffer) {
-#pragma unroll
-        for (int j = 0; j < kPieces; ++j) {
-            xs_flat[buffer * kBufferStride + piece_dst[j]] = stage[j];
+        for (int j = 0; j < kFrags; ++j) {
+            const int f = wave * kFrags + j;
+            if ((f >> 2) < live_tiles) {
+                __builtin_amdgcn_global_load_lds(
+                    (const AEON_GLOBAL void*)(frag_src[j] + g * 128),
+                    (__attribute__((address_space(3))) void*)(xs_flat + buffer * kBufferStride + f * 64),
+                    16, 0, 0);
+            }
         }
     };
 
-    fetch_tile(0);
+    fetch_tile(0, 0);
     load_weights(0);
-    publish_tile(0);
+    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
 
     for (int g = 0; g < groups; ++g) {
@@ -140,7 +145,7 @@ __global__ __launch_bounds__(256) void a64_grouped_kernel(SegGateUpArgs gu, SegD
                 v.u = sc[m][r];
                 scur[m][r] = half2_t{v.h, v.h};
             }
-        fetch_tile(gn);
+        fetch_tile(gn, (g + 1) & 1);
         load_weights(gn);
         const half8_t* xb = xs_flat + (g & 1) * kBufferStride;
 #pragma unroll
@@ -164,7 +169,7 @@ __global__ __launch_bounds__(256) void a64_grouped_kernel(SegGateUpArgs gu, SegD
                 }
             }
         }
-        publish_tile((g + 1) & 1);
+        __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
     }
 

@@ -5,6 +5,7 @@
 // their upper bounds and workgroups past the live count exit at once.
 #include "expert_a64.hpp"
 #include "permutation.hpp"
+#include "router.hpp"
 
 #include <cstdlib>
 
@@ -224,17 +225,19 @@ extern "C" int aeon_moe_layer_decode(const aeon_moe_layer* layer, const void* d_
     const LayerWorkspace w = carve(*layer, tokens, d_workspace);
     AEON_REQUIRE(workspace_bytes >= w.bytes, AEON_ERR_INVALID_ARGUMENT,
                  "%s: workspace of %zu bytes, %zu needed", who, workspace_bytes, w.bytes);
-    if (int rc = aeon_router_logits(d_x, x_stride, layer->d_router_weight, w.logits, tokens,
-                                    layer->hidden, layer->experts, w.logits_partial,
-                                    aeon_router_logits_workspace_bytes(tokens, layer->hidden,
-                                                                       layer->experts),
-                                    stream)) {
+    AEON_REQUIRE(layer->score_kind == AEON_ROUTER_SCORE_SQRT_SOFTPLUS ||
+                     layer->score_kind == AEON_ROUTER_SCORE_SIGMOID,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: unknown score kind %d", who, layer->score_kind);
+    hipStream_t s = as_stream(stream);
+    if (int rc = launch_router_partials(d_x, x_stride, layer->d_router_weight, w.logits_partial,
+                                        tokens, layer->hidden, layer->experts, s)) {
         return rc;
     }
-    if (int rc = aeon_moe_router(w.logits, layer->d_router_bias, nullptr, nullptr, d_topk_weights,
-                                 d_topk_ids, tokens, layer->experts, layer->top_k,
-                                 layer->routed_scaling_factor, layer->renormalize,
-                                 layer->score_kind, stream)) {
+    if (int rc = launch_router_topk(w.logits_partial, router_logits_chunks(tokens, layer->hidden),
+                                    w.logits, layer->d_router_bias, nullptr, nullptr,
+                                    d_topk_weights, d_topk_ids, tokens, layer->experts,
+                                    layer->top_k, layer->routed_scaling_factor, layer->renormalize,
+                                    layer->score_kind, s)) {
         return rc;
     }
     return aeon_moe_layer_routed(layer, d_x, x_stride, tokens, d_topk_ids, d_topk_weights, d_out,

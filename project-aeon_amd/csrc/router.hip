@@ -4,107 +4,127 @@
 // host computation (descending biased score, ties to the lower index); two experts whose
 // biased scores differ by less than an fp32 rounding would otherwise be ordered by rounding
 // noise, and the routed ids have to match the host bit for bit.
-#include "common.hpp"
+#include "router.hpp"
 
 namespace aeon355 {
 
-constexpr int kRouterTokenTile = 16;
+constexpr int kRouterTokenTile = 16;   // tokens per workgroup: the M of the fp32 MFMA
+constexpr int kRouterWaves = 8;        // waves per workgroup, each with its own slice of rows
+constexpr int kRouterWaveRows = 112;   // rows of Wr per wave (7 MFMA passes of 16 rows)
+constexpr int kRouterChunkRows = kRouterWaves * kRouterWaveRows;  // rows per workgroup
 constexpr int kRouterMaxExperts = 1024;
 
-// partial[c][t][e] = sum over the rows h of chunk c of x[t][h] * Wr[h][e].
-// One workgroup = (chunk, tile of 16 tokens), four waves. A wave takes every fourth row of the
-// chunk and reads it as one coalesced float4-per-lane load (64 lanes x 4 experts = 256 experts
-// per pass), eight rows in flight; the four waves' sums meet in LDS in wave order, so the
-// result does not depend on timing.
-__global__ __launch_bounds__(256) void router_logits_partial_kernel(
+// partial[c][t][e] = sum over the rows h of chunk c of x[t][h] * Wr[h][e], on the fp32 matrix
+// cores (v_mfma_f32_16x16x4_f32: full fp32 operands and accumulate).
+// One workgroup = (chunk of 896 rows, 16 tokens, 64 experts). Each of its eight waves takes 112
+// rows; per 16 rows a lane reads 4 activations (8 bytes) and four float4 of Wr (row
+// 4*(l/16)+s, experts 4*(l%16)..+3 of the block -- 256 contiguous bytes per row), which feed
+// 16 MFMAs: component j of the float4 is the B operand of the tile holding experts 4n+j. The
+// waves' tiles are added through LDS in wave order, so the result does not depend on timing.
+__global__ __launch_bounds__(kRouterWaves * 64) void router_logits_partial_kernel(
     const uint16_t* __restrict__ x, long x_stride, const float* __restrict__ wr,
-    float* __restrict__ partial, int tokens, int hidden, int experts, int chunk_rows) {
+    float* __restrict__ partial, int tokens, int hidden, int experts) {
     const int chunk = blockIdx.x;
     const int t0 = blockIdx.y * kRouterTokenTile;
-    const int h0 = chunk * chunk_rows;
-    const int h1 = min(hidden, h0 + chunk_rows);
+    const int e0 = blockIdx.z * 64;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    extern __shared__ float lds[];
-    float* xs = lds;                                  // [chunk_rows][kRouterTokenTile]
-    float* sums = lds + chunk_rows * kRouterTokenTile;  // [3][kRouterTokenTile][256]: waves 1..3
-    for (int i = threadIdx.x; i < kRouterTokenTile * chunk_rows; i += blockDim.x) {
-        const int t = i % kRouterTokenTile;
-        const int h = h0 + i / kRouterTokenTile;
-        xs[i] = (t0 + t < tokens && h < h1) ? half_bits_to_float(x[(t0 + t) * x_stride + h]) : 0.0f;
+    const int n = lane & 15;
+    const int kq = lane >> 4;
+    const int h_begin = chunk * kRouterChunkRows + wave * kRouterWaveRows;
+    const int token = min(t0 + n, tokens - 1);  // a padded row repeats a live token, never stored
+    const uint16_t* xrow = x + token * x_stride;
+    const int e = e0 + 4 * n;
+
+    float4_t acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    // every load of the wave's 112 rows is issued before the first MFMA: the kernel is a few
+    // microseconds long, so one round trip to HBM is all it can afford
+    constexpr int kSteps = kRouterWaveRows / 16;
+    uint2 xa[kSteps];
+    float4_t b[kSteps][4];
+    const bool whole = (e + 3 < experts) && (h_begin + kRouterWaveRows <= hidden) && (x_stride % 4 == 0);
+    if (whole) {
+#pragma unroll
+        for (int step = 0; step < kSteps; ++step) {
+            const int h = h_begin + step * 16 + 4 * kq;
+            xa[step] = *reinterpret_cast<const uint2*>(xrow + h);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                b[step][r] = *reinterpret_cast<const float4_t*>(wr + static_cast<size_t>(h + r) * experts + e);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int step = 0; step < kSteps; ++step) {
+            const int h = h_begin + step * 16 + 4 * kq;
+            uint16_t xv[4] = {0, 0, 0, 0};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                b[step][r] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                if (h + r < hidden) {
+                    xv[r] = xrow[h + r];
+                    for (int q = 0; q < 4; ++q) {
+                        if (e + q < experts) b[step][r][q] = wr[static_cast<size_t>(h + r) * experts + e + q];
+                    }
+                }
+            }
+            xa[step] = make_uint2(xv[0] | (static_cast<uint32_t>(xv[1]) << 16),
+                                  xv[2] | (static_cast<uint32_t>(xv[3]) << 16));
+        }
+    }
+#pragma unroll
+    for (int step = 0; step < kSteps; ++step) {
+        const float a[4] = {half_bits_to_float(static_cast<uint16_t>(xa[step].x & 0xFFFFu)),
+                            half_bits_to_float(static_cast<uint16_t>(xa[step].x >> 16)),
+                            half_bits_to_float(static_cast<uint16_t>(xa[step].y & 0xFFFFu)),
+                            half_bits_to_float(static_cast<uint16_t>(xa[step].y >> 16))};
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[r], b[step][r][j], acc[j], 0, 0, 0);
+            }
+    }
+
+    __shared__ float4_t sums[kRouterWaves - 1][4][64];
+    if (wave > 0) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sums[wave - 1][j][lane] = acc[j];
     }
     __syncthreads();
-    for (int e0 = 0; e0 < experts; e0 += 256) {
-        const int e = e0 + lane * 4;
-        float4_t acc[kRouterTokenTile];
+    if (wave == 0) {
 #pragma unroll
-        for (int t = 0; t < kRouterTokenTile; ++t) acc[t] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-        constexpr int kRows = 8;
-        for (int hb = h0 + wave; hb < h1; hb += 4 * kRows) {
-            float4_t w[kRows];
+        for (int j = 0; j < 4; ++j) {
+            float4_t v = acc[j];
 #pragma unroll
-            for (int j = 0; j < kRows; ++j) {
-                const int h = hb + 4 * j;
-                w[j] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-                if (h < h1 && e + 3 < experts) {
-                    w[j] = *reinterpret_cast<const float4_t*>(wr + static_cast<size_t>(h) * experts + e);
-                } else if (h < h1) {
-                    for (int q = 0; q < 4; ++q) {
-                        if (e + q < experts) w[j][q] = wr[static_cast<size_t>(h) * experts + e + q];
-                    }
-                }
-            }
+            for (int w = 0; w < kRouterWaves - 1; ++w) v += sums[w][j][lane];
+            // lane holds tokens 4*kq + i (i = 0..3) of expert e0 + 4*n + j
+            const int ee = e0 + 4 * n + j;
 #pragma unroll
-            for (int j = 0; j < kRows; ++j) {
-                const int h = hb + 4 * j;
-                if (h < h1) {
-                    const float* xrow = xs + (h - h0) * kRouterTokenTile;
-#pragma unroll
-                    for (int t = 0; t < kRouterTokenTile; ++t) acc[t] += xrow[t] * w[j];
+            for (int i = 0; i < 4; ++i) {
+                const int t = t0 + 4 * kq + i;
+                if (t < tokens && ee < experts) {
+                    partial[(static_cast<size_t>(chunk) * tokens + t) * experts + ee] = v[i];
                 }
             }
         }
-        if (wave > 0) {
-#pragma unroll
-            for (int t = 0; t < kRouterTokenTile; ++t) {
-                *reinterpret_cast<float4_t*>(sums + ((wave - 1) * kRouterTokenTile + t) * 256 +
-                                             lane * 4) = acc[t];
-            }
-        }
-        __syncthreads();
-        if (wave == 0) {
-#pragma unroll
-            for (int t = 0; t < kRouterTokenTile; ++t) {
-                float4_t v = acc[t];
-#pragma unroll
-                for (int w2 = 0; w2 < 3; ++w2) {
-                    v += *reinterpret_cast<const float4_t*>(sums + (w2 * kRouterTokenTile + t) * 256 +
-                                                            lane * 4);
-                }
-                if (t0 + t < tokens) {
-                    float* dst = partial + (static_cast<size_t>(chunk) * tokens + t0 + t) * experts + e;
-                    for (int q = 0; q < 4; ++q) {
-                        if (e + q < experts) dst[q] = v[q];
-                    }
-                }
-            }
-        }
-        __syncthreads();
     }
 }
 
-// logits[i] = sum over chunks, ascending (eight loads in flight).
+// logits[i] = sum over chunks, ascending (sixteen loads in flight).
 __global__ __launch_bounds__(256) void router_logits_reduce_kernel(
     const float* __restrict__ partial, float* __restrict__ logits, int chunks, size_t count) {
     const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= count) return;
     float acc = 0.0f;
-    for (int c0 = 0; c0 < chunks; c0 += 8) {
-        float v[8];
+    for (int c0 = 0; c0 < chunks; c0 += 16) {
+        float v[16];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = c0 + j < chunks ? partial[static_cast<size_t>(c0 + j) * count + i] : 0.0f;
+        for (int j = 0; j < 16; ++j) v[j] = c0 + j < chunks ? partial[static_cast<size_t>(c0 + j) * count + i] : 0.0f;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc += v[j];
+        for (int j = 0; j < 16; ++j) acc += v[j];
     }
     logits[i] = acc;
 }
@@ -115,98 +135,126 @@ __device__ __forceinline__ double router_score(double logit, int score_kind) {
     return sqrt(softplus);
 }
 
-// One wave per token. Lane l owns experts l, l+64, ...; each of the k rounds is a lane-local
-// scan in ascending index followed by a wave arg-max whose ties go to the lower index.
-template <int kPerLane>
-__global__ __launch_bounds__(64) void router_topk_kernel(
-    const float* __restrict__ logits, const float* __restrict__ bias,
-    const int64_t* __restrict__ hash_table, const int32_t* __restrict__ token_ids,
-    float* __restrict__ topk_weights, int32_t* __restrict__ topk_indices, int experts, int top_k,
-    float scaling, int renormalize, int score_kind) {
+// One workgroup of 256 threads per token. When `partial` is given the threads first sum the
+// token's logits over the chunks (ascending) into `logits`. Every thread then scores its experts
+// in fp64 and finds each one's rank under the total order (biased score descending, index
+// ascending) by comparing against all experts held in LDS: rank r < top_k is the r-th pick.
+// No serial scan and no cross-lane argmax, and the order -- ties to the lower index included --
+// is exactly the specification's.
+template <int kPerThread>
+__global__ __launch_bounds__(256) void router_topk_kernel(
+    const float* __restrict__ partial, int chunks, int tokens, float* __restrict__ logits,
+    const float* __restrict__ bias, const int64_t* __restrict__ hash_table,
+    const int32_t* __restrict__ token_ids, float* __restrict__ topk_weights,
+    int32_t* __restrict__ topk_indices, int experts, int top_k, float scaling, int renormalize,
+    int score_kind) {
     const int token = blockIdx.x;
-    const int lane = threadIdx.x;
-    const float* row = logits + static_cast<size_t>(token) * experts;
-
-    double score[kPerLane];
-    double choice[kPerLane];
-#pragma unroll
-    for (int j = 0; j < kPerLane; ++j) {
-        const int e = lane + 64 * j;
-        if (e < experts) {
-            score[j] = router_score(static_cast<double>(row[e]), score_kind);
-            choice[j] = bias != nullptr ? score[j] + static_cast<double>(bias[e]) : score[j];
-        } else {
-            score[j] = 0.0;
-            choice[j] = -1.0e300;
-        }
-    }
-
+    __shared__ double choice_lds[kPerThread * 256];
+    __shared__ double score_lds[kPerThread * 256];
     __shared__ double picked_score[64];
     __shared__ int picked_id[64];
-    const bool hashed = hash_table != nullptr && token_ids != nullptr;
-    for (int k = 0; k < top_k; ++k) {
-        int best_e;
-        if (hashed) {
-            best_e = static_cast<int>(hash_table[static_cast<size_t>(token_ids[token]) * top_k + k]);
-        } else {
-            double best_v = -1.0e300;
-            best_e = 0x7FFFFFFF;
+    float* out_row = logits + static_cast<size_t>(token) * experts;
+    double my_choice[kPerThread];
 #pragma unroll
-            for (int j = 0; j < kPerLane; ++j) {
-                const int e = lane + 64 * j;
-                if (e < experts && choice[j] > best_v) {
-                    best_v = choice[j];
-                    best_e = e;
-                }
-            }
+    for (int j = 0; j < kPerThread; ++j) {
+        const int e = threadIdx.x + 256 * j;
+        my_choice[j] = -1.0e300;
+        if (e < experts) {
+            float acc;
+            if (partial != nullptr) {
+                acc = 0.0f;
+                const size_t count = static_cast<size_t>(tokens) * experts;
+                const float* p = partial + static_cast<size_t>(token) * experts + e;
+                for (int c0 = 0; c0 < chunks; c0 += 16) {
+                    float v[16];
 #pragma unroll
-            for (int offset = 32; offset > 0; offset >>= 1) {
-                const double other_v = __shfl_xor(best_v, offset, 64);
-                const int other_e = __shfl_xor(best_e, offset, 64);
-                if (other_v > best_v || (other_v == best_v && other_e < best_e)) {
-                    best_v = other_v;
-                    best_e = other_e;
-                }
-            }
-        }
-        // the owner publishes the unbiased score and retires the expert
-        if ((best_e & 63) == lane) {
-            const int j = best_e >> 6;
-            double s = 0.0;
+                    for (int q = 0; q < 16; ++q) v[q] = c0 + q < chunks ? p[static_cast<size_t>(c0 + q) * count] : 0.0f;
 #pragma unroll
-            for (int jj = 0; jj < kPerLane; ++jj) {
-                if (jj == j) {
-                    s = score[jj];
-                    if (!hashed) choice[jj] = -1.0e300;
+                    for (int q = 0; q < 16; ++q) acc += v[q];
                 }
+                out_row[e] = acc;
+            } else {
+                acc = out_row[e];
             }
-            picked_score[k] = s;
-            picked_id[k] = best_e;
+            const double sc = router_score(static_cast<double>(acc), score_kind);
+            my_choice[j] = bias != nullptr ? sc + static_cast<double>(bias[e]) : sc;
+            score_lds[e] = sc;
+            choice_lds[e] = my_choice[j];
         }
     }
     __syncthreads();
-    if (lane < top_k) {
+
+    const bool hashed = hash_table != nullptr && token_ids != nullptr;
+    if (hashed) {
+        if (threadIdx.x < top_k) {
+            const int e = static_cast<int>(
+                hash_table[static_cast<size_t>(token_ids[token]) * top_k + threadIdx.x]);
+            picked_id[threadIdx.x] = e;
+            picked_score[threadIdx.x] = score_lds[e];
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < kPerThread; ++j) {
+            const int e = threadIdx.x + 256 * j;
+            if (e < experts) {
+                int rank = 0;
+                const double mine = my_choice[j];
+                for (int f = 0; f < experts; ++f) {
+                    const double other = choice_lds[f];
+                    rank += (other > mine || (other == mine && f < e)) ? 1 : 0;
+                }
+                if (rank < top_k) {
+                    picked_id[rank] = e;
+                    picked_score[rank] = score_lds[e];
+                }
+            }
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < top_k) {
         double sum = 0.0;
         for (int k = 0; k < top_k; ++k) sum += picked_score[k];
-        double w = picked_score[lane];
+        double w = picked_score[threadIdx.x];
         if (renormalize) w = w / (sum + 1e-20);
         w *= static_cast<double>(scaling);
-        topk_indices[static_cast<size_t>(token) * top_k + lane] = picked_id[lane];
-        topk_weights[static_cast<size_t>(token) * top_k + lane] = static_cast<float>(w);
+        topk_indices[static_cast<size_t>(token) * top_k + threadIdx.x] = picked_id[threadIdx.x];
+        topk_weights[static_cast<size_t>(token) * top_k + threadIdx.x] = static_cast<float>(w);
     }
 }
 
 int router_logits_chunks(int tokens, int hidden) {
-    // about 256 workgroups: many short chunks for a decode batch, few for a prefill chunk
+    (void)tokens;
+    return (hidden + kRouterChunkRows - 1) / kRouterChunkRows;
+}
+
+// Launches the partial-sum kernel; the chunk sums are left for the caller's reduce.
+int launch_router_partials(const void* d_x, int x_stride, const float* d_router_weight,
+                           float* partial, int tokens, int hidden, int experts,
+                           hipStream_t stream) {
+    const int chunks = router_logits_chunks(tokens, hidden);
     const int tiles = (tokens + kRouterTokenTile - 1) / kRouterTokenTile;
-    int chunks = 256 / (tiles > 0 ? tiles : 1);
-    if (chunks > 64) chunks = 64;
-    if (chunks < 1) chunks = 1;
-    const int max_chunks = (hidden + 31) / 32;
-    if (chunks > max_chunks) chunks = max_chunks;
-    const int min_chunks = (hidden + 127) / 128;  // a chunk's activations must fit in LDS
-    if (chunks < min_chunks) chunks = min_chunks;
-    return chunks;
+    router_logits_partial_kernel<<<dim3(chunks, tiles, (experts + 63) / 64), kRouterWaves * 64, 0,
+                                   stream>>>(static_cast<const uint16_t*>(d_x), x_stride,
+                                             d_router_weight, partial, tokens, hidden, experts);
+    AEON_LAUNCH_CHECK();
+    return AEON_OK;
+}
+
+int launch_router_topk(const float* partial, int chunks, float* logits, const float* bias,
+                       const int64_t* hash_table, const int32_t* token_ids, float* topk_weights,
+                       int32_t* topk_indices, int tokens, int experts, int top_k, float scaling,
+                       int renormalize, int score_kind, hipStream_t stream) {
+    if (experts <= 256) {
+        router_topk_kernel<1><<<tokens, 256, 0, stream>>>(
+            partial, chunks, tokens, logits, bias, hash_table, token_ids, topk_weights,
+            topk_indices, experts, top_k, scaling, renormalize, score_kind);
+    } else {
+        router_topk_kernel<kRouterMaxExperts / 256><<<tokens, 256, 0, stream>>>(
+            partial, chunks, tokens, logits, bias, hash_table, token_ids, topk_weights,
+            topk_indices, experts, top_k, scaling, renormalize, score_kind);
+    }
+    AEON_LAUNCH_CHECK();
+    return AEON_OK;
 }
 
 }  // namespace aeon355
@@ -232,17 +280,12 @@ extern "C" int aeon_router_logits(const void* d_x, int x_stride, const float* d_
                  AEON_ERR_INVALID_ARGUMENT, "%s: workspace of %zu bytes is too small", who,
                  workspace_bytes);
     const int chunks = router_logits_chunks(tokens, hidden);
-    const int chunk_rows = (hidden + chunks - 1) / chunks;
-    const int tiles = (tokens + kRouterTokenTile - 1) / kRouterTokenTile;
-    const size_t lds = static_cast<size_t>(kRouterTokenTile) * (chunk_rows + 3 * 256) * sizeof(float);
-    AEON_REQUIRE(lds <= 64 * 1024, AEON_ERR_INVALID_ARGUMENT,
-                 "%s: hidden=%d needs %zu bytes of LDS per chunk", who, hidden, lds);
     hipStream_t s = as_stream(stream);
     float* partial = static_cast<float*>(d_workspace);
-    router_logits_partial_kernel<<<dim3(chunks, tiles), 256, lds, s>>>(
-        static_cast<const uint16_t*>(d_x), x_stride, d_router_weight, partial, tokens, hidden,
-        experts, chunk_rows);
-    AEON_LAUNCH_CHECK();
+    if (int rc = launch_router_partials(d_x, x_stride, d_router_weight, partial, tokens, hidden,
+                                        experts, s)) {
+        return rc;
+    }
     const size_t count = static_cast<size_t>(tokens) * experts;
     router_logits_reduce_kernel<<<static_cast<unsigned>((count + 255) / 256), 256, 0, s>>>(
         partial, d_logits, chunks, count);
@@ -267,15 +310,9 @@ extern "C" int aeon_moe_router(const float* d_logits, const float* d_bias,
     AEON_REQUIRE((d_hash_table == nullptr) == (d_token_ids == nullptr), AEON_ERR_INVALID_ARGUMENT,
                  "%s: the hash branch needs both the table and the token ids", who);
     if (tokens == 0) return AEON_OK;
-    if (experts <= 256) {
-        router_topk_kernel<4><<<tokens, 64, 0, as_stream(stream)>>>(
-            d_logits, d_bias, d_hash_table, d_token_ids, d_topk_weights, d_topk_indices, experts,
-            top_k, routed_scaling_factor, renormalize, score_kind);
-    } else {
-        router_topk_kernel<kRouterMaxExperts / 64><<<tokens, 64, 0, as_stream(stream)>>>(
-            d_logits, d_bias, d_hash_table, d_token_ids, d_topk_weights, d_topk_indices, experts,
-            top_k, routed_scaling_factor, renormalize, score_kind);
-    }
-    AEON_LAUNCH_CHECK();
-    return AEON_OK;
+    // with no partial sums the kernel only reads `logits`
+    return launch_router_topk(nullptr, 0, const_cast<float*>(d_logits), d_bias, d_hash_table,
+                              d_token_ids, d_topk_weights, d_topk_indices, tokens, experts, top_k,
+                              routed_scaling_factor, renormalize, score_kind, as_stream(stream));
 }
+
