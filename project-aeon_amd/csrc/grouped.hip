@@ -31,150 +31,183 @@ __device__ __forceinline__ half8_t scaled_fragment(uint32_t word, half2_t scale2
     return v;
 }
 
-template <bool GATE_UP, int R>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void a64_grouped_kernel(
-    SegGateUpArgs gu, SegDownArgs dn) {
-    constexpr int NM = GATE_UP ? 2 : 1;
-    constexpr int MT = kGroupedMT;
-    const SegmentList& seg = GATE_UP ? gu.seg : dn.seg;
-    const int s = blockIdx.y;
-    if (s >= *seg.total) return;
-    const int first = seg.first[s];
-    const int count = seg.count[s];
-    const aeon_a64_expert e = (GATE_UP ? gu.experts : dn.experts)[seg.expert[s]];
+// s_waitcnt that only bounds the number of outstanding vector-memory loads (gfx9 encoding:
+// vmcnt in bits 3:0 and 15:14, the export and LDS/scalar counters left at "no wait").
+#define AEON_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | 0x0F70)
 
+// The body for a window of LIVE token tiles (LIVE is the tile's live count rounded up to a power
+// of two; rows past the count are clamped reads whose results are never stored), with the
+// weights and the activation window of DEPTH later K groups in flight while one is computed.
+//
+// Windows with few tokens are bound by the latency of the weight stream, not by arithmetic: they
+// have few accumulators, so the registers (and the LDS a small window leaves free) go into a deep
+// ring instead. A full window is MFMA-bound, re-reads weights its neighbour tiles have just
+// pulled into L2, and keeps one group in flight.
+//
+// Inside a K step everything is straight-line code: the B fragments of an MFMA step are requested
+// together and the next step's weight fragments are unpacked while the current step's MFMAs run.
+// Loads complete in issue order and every K step issues the same number, so "the window of the
+// next group has landed" is a bound on the count of outstanding loads. The step ends in a bare
+// s_barrier: a wave arrives only after its own window requests have landed in LDS and after it
+// has consumed its reads of the slot about to be overwritten, which is all the ordering the
+// ring needs (the fences of __syncthreads would drain the whole ring every step).
+template <bool GATE_UP, int R, int LIVE, int DEPTH>
+__device__ __forceinline__ void grouped_run(const SegGateUpArgs& gu, const SegDownArgs& dn,
+                                            const aeon_a64_expert& e, int first, int count,
+                                            half8_t* xs_flat) {
+    constexpr int NM = GATE_UP ? 2 : 1;
+    constexpr int STAGES = DEPTH + 1;
+    constexpr int kBufferStride = LIVE * 4 * 64;  // in 16-byte units
+    constexpr int kLoadsPerStep = LIVE + NM * R * 2;
+    constexpr int kInFlight = (DEPTH - 1) * kLoadsPerStep;
+    static_assert(STAGES * LIVE <= 2 * kGroupedMT, "ring must fit the window buffer");
+    static_assert(kInFlight < 64, "vmcnt is a 6-bit counter");
+    constexpr bool kOverlapUnpack = true;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int n = lane & 15;
     const int chunk = lane >> 4;
     const int tile0 = (blockIdx.x * 4 + wave) * R;
-    const int live_tiles = (count + 15) >> 4;
 
     const int K = GATE_UP ? gu.H : dn.I;
     const int groups = K / 128;
-    const AEON_GLOBAL u32x4_t* pm[NM];
-    const AEON_GLOBAL uint16_t* sm[NM];
-    pm[0] = as_global<u32x4_t>(GATE_UP ? e.w1_packed : e.w2_packed);
-    sm[0] = as_global<uint16_t>(GATE_UP ? e.w1_scale : e.w2_scale);
+    // Uniform base + 32-bit lane offset addressing keeps the address registers few.
+    const AEON_GLOBAL char* pm[NM];
+    const AEON_GLOBAL char* sm[NM];
+    pm[0] = as_global<char>(GATE_UP ? e.w1_packed : e.w2_packed);
+    sm[0] = as_global<char>(GATE_UP ? e.w1_scale : e.w2_scale);
     if (GATE_UP) {
-        pm[NM - 1] = as_global<u32x4_t>(e.w3_packed);
-        sm[NM - 1] = as_global<uint16_t>(e.w3_scale);
+        pm[NM - 1] = as_global<char>(e.w3_packed);
+        sm[NM - 1] = as_global<char>(e.w3_scale);
+    }
+    uint32_t woff[R], soff[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const uint32_t t = static_cast<uint32_t>(tile0 + r) * groups;
+        woff[r] = (t * 64 + lane) * 16;
+        soff[r] = (t * 16 + n) * 2;  // the A operand's row is lane % 16
     }
 
-    // Activation tile in LDS, fragment-major: [buffer][token tile][step][lane] x 16 bytes, so a
-    // B operand is one conflict-free ds_read_b128 per lane.
-    __shared__ half8_t xs[2][MT][4][64];
-
-    // Staging assignment: the tile is MT*4 fragments of 1 KiB (token tile mt, MFMA step st); wave
-    // w stages fragments w*kFrags .. +kFrags-1. Lane (n, chunk) of a fragment fetches 16 bytes of
-    // row mt*16+n at column st*32 + chunk*8 and stores them at the lane's own 16-byte slot, so
-    // the LDS write of a wave is one contiguous KiB (no bank conflicts) and is the exact image
-    // the B-operand read wants.
-    constexpr int kFrags = MT * 4 / 4;  // per wave
-    const AEON_GLOBAL uint16_t* frag_src[kFrags];
+    // Staging: the window is LIVE*4 fragments of 1 KiB (token tile j, MFMA step st); wave w
+    // stages step w of every token tile. Lane (n, chunk) of a fragment fetches 16 bytes of row
+    // j*16+n at column w*32 + chunk*8 straight into its own 16-byte slot of the fragment
+    // (global_load_lds), which is the exact image the B-operand read wants.
+    const AEON_GLOBAL char* xbase = as_global<char>(GATE_UP ? static_cast<const void*>(gu.x)
+                                                            : static_cast<const void*>(dn.hidden));
+    uint32_t xoff[LIVE];
 #pragma unroll
-    for (int j = 0; j < kFrags; ++j) {
-        const int f = wave * kFrags + j;
-        const int row = (f >> 2) * 16 + n;
+    for (int j = 0; j < LIVE; ++j) {
+        const int row = j * 16 + n;
         const int live_row = row < count ? row : count - 1;
         const int position = first + live_row;
-        const int column = (f & 3) * 32 + chunk * 8;
+        const int column = wave * 32 + chunk * 8;
         if (GATE_UP) {
             const long src_row = gu.row_index != nullptr ? gu.row_index[position] : position;
-            frag_src[j] = as_global<uint16_t>(gu.x) + src_row * gu.x_stride + column;
+            xoff[j] = static_cast<uint32_t>((src_row * gu.x_stride + column) * 2);
         } else {
-            frag_src[j] = as_global<uint16_t>(dn.hidden) + static_cast<size_t>(position) * dn.I + column;
+            xoff[j] = static_cast<uint32_t>((static_cast<size_t>(position) * dn.I + column) * 2);
         }
     }
-    half8_t* xs_flat = &xs[0][0][0][0];
-    constexpr int kBufferStride = MT * 4 * 64;
 
-    float4_t acc[NM][R][MT];
+    float4_t acc[NM][R][LIVE];
 #pragma unroll
     for (int m = 0; m < NM; ++m)
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) acc[m][r][mt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+            for (int mt = 0; mt < LIVE; ++mt) acc[m][r][mt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-    u32x4_t wq[NM][R];
-    uint16_t sc[NM][R];
-    auto load_weights = [&](int g) {
-#pragma unroll
-        for (int m = 0; m < NM; ++m)
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const size_t t = static_cast<size_t>(tile0 + r) * groups + g;
-                wq[m][r] = pm[m][t * 64 + lane];
-                sc[m][r] = sm[m][t * 16 + n];  // the A operand's row is lane % 16
-            }
-    };
+    u32x4_t wq[STAGES][NM][R];
+    uint16_t sc[STAGES][NM][R];
 
-    // Activation fragments go from global memory straight into LDS (global_load_lds, 16 bytes
-    // per lane landing at the lane's own slot of the fragment): no staging registers, no LDS
-    // write instructions. The tile for group g+1 is requested at the top of step g into the
-    // other buffer; every wave drains its own requests before the barrier that ends the step.
-    auto fetch_tile = [&](int g, int buffer) {
-#pragma unroll
-        for (int j = 0; j < kFrags; ++j) {
-            const int f = wave * kFrags + j;
-            if ((f >> 2) < live_tiles) {
-                __builtin_amdgcn_global_load_lds(
-                    (const AEON_GLOBAL void*)(frag_src[j] + g * 128),
-                    (__attribute__((address_space(3))) void*)(xs_flat + buffer * kBufferStride + f * 64),
-                    16, 0, 0);
-            }
-        }
-    };
+    // Requests for K group g (clamped to the last one so every step issues the same count; the
+    // clamped repeats land in ring slots nobody reads again).
+#define AEON_GROUPED_ISSUE(g_, stage_)                                                              \
+    do {                                                                                            \
+        const int gi_ = (g_) < groups ? (g_) : groups - 1;                                          \
+        _Pragma("unroll") for (int j = 0; j < LIVE; ++j) {                                          \
+            __builtin_amdgcn_global_load_lds(                                                       \
+                (const AEON_GLOBAL void*)(xbase + (xoff[j] + static_cast<uint32_t>(gi_) * 256u)),   \
+                (__attribute__((address_space(3))) void*)(xs_flat + (stage_) * kBufferStride +      \
+                                                          (j * 4 + wave) * 64),                     \
+                16, 0, 0);                                                                          \
+        }                                                                                           \
+        _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                            \
+            _Pragma("unroll") for (int r = 0; r < R; ++r) {                                         \
+                wq[stage_][m][r] = *(const AEON_GLOBAL u32x4_t*)(                                   \
+                    pm[m] + (woff[r] + static_cast<uint32_t>(gi_) * 1024u));                        \
+                sc[stage_][m][r] = *(const AEON_GLOBAL uint16_t*)(                                  \
+                    sm[m] + (soff[r] + static_cast<uint32_t>(gi_) * 32u));                          \
+            }                                                                                       \
+        }                                                                                           \
+    } while (0)
 
-    fetch_tile(0, 0);
-    load_weights(0);
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < DEPTH; ++s) AEON_GROUPED_ISSUE(s, s);
+    AEON_WAIT_VMCNT(kInFlight);
+    __builtin_amdgcn_s_barrier();
 
-    for (int g = 0; g < groups; ++g) {
-        const int gn = g + 1 < groups ? g + 1 : g;  // the last step refetches its own group, unused
-        u32x4_t wcur[NM][R];
-        half2_t scur[NM][R];
+    for (int g0 = 0; g0 < groups; g0 += STAGES) {
 #pragma unroll
-        for (int m = 0; m < NM; ++m)
+        for (int s = 0; s < STAGES; ++s) {
+            const int g = g0 + s;
+            if (g < groups) {
+                AEON_GROUPED_ISSUE(g + DEPTH, (s + DEPTH) % STAGES);
+                half2_t scur[NM][R];
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                wcur[m][r] = wq[m][r];
-                union { uint16_t u; half_t h; } v;
-                v.u = sc[m][r];
-                scur[m][r] = half2_t{v.h, v.h};
-            }
-        fetch_tile(gn, (g + 1) & 1);
-        load_weights(gn);
-        const half8_t* xb = xs_flat + (g & 1) * kBufferStride;
+                for (int m = 0; m < NM; ++m)
 #pragma unroll
-        for (int st = 0; st < 4; ++st) {
-            half8_t a[NM][R];
+                    for (int r = 0; r < R; ++r) {
+                        union { uint16_t u; half_t h; } v;
+                        v.u = sc[s][m][r];
+                        scur[m][r] = half2_t{v.h, v.h};
+                    }
+                const half8_t* xb = xs_flat + s * kBufferStride;
+                half8_t a[NM][R];
 #pragma unroll
-            for (int m = 0; m < NM; ++m)
+                for (int m = 0; m < NM; ++m)
 #pragma unroll
-                for (int r = 0; r < R; ++r) a[m][r] = scaled_fragment(wcur[m][r][st], scur[m][r]);
+                    for (int r = 0; r < R; ++r) a[m][r] = scaled_fragment(wq[s][m][r][0], scur[m][r]);
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                if (mt < live_tiles) {
-                    const half8_t b = xb[(mt * 4 + st) * 64 + lane];
+                for (int st = 0; st < 4; ++st) {
+                    half8_t b[LIVE];
 #pragma unroll
-                    for (int m = 0; m < NM; ++m)
+                    for (int mt = 0; mt < LIVE; ++mt) b[mt] = xb[(mt * 4 + st) * 64 + lane];
+                    half8_t a_next[NM][R];
+                    if (kOverlapUnpack && st < 3) {
 #pragma unroll
-                        for (int r = 0; r < R; ++r) {
-                            acc[m][r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                a[m][r], b, acc[m][r][mt], 0, 0, 0);
-                        }
+                        for (int m = 0; m < NM; ++m)
+#pragma unroll
+                            for (int r = 0; r < R; ++r)
+                                a_next[m][r] = scaled_fragment(wq[s][m][r][st < 3 ? st + 1 : 3], scur[m][r]);
+                    }
+#pragma unroll
+                    for (int mt = 0; mt < LIVE; ++mt)
+#pragma unroll
+                        for (int m = 0; m < NM; ++m)
+#pragma unroll
+                            for (int r = 0; r < R; ++r)
+                                acc[m][r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                    a[m][r], b[mt], acc[m][r][mt], 0, 0, 0);
+                    if (st < 3) {
+#pragma unroll
+                        for (int m = 0; m < NM; ++m)
+#pragma unroll
+                            for (int r = 0; r < R; ++r)
+                                a[m][r] = kOverlapUnpack
+                                              ? a_next[m][r]
+                                              : scaled_fragment(wq[s][m][r][st < 3 ? st + 1 : 3], scur[m][r]);
+                    }
                 }
+                AEON_WAIT_VMCNT(kInFlight);
+                __builtin_amdgcn_s_barrier();
             }
         }
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
     }
+#undef AEON_GROUPED_ISSUE
 
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
+    for (int mt = 0; mt < LIVE; ++mt) {
         const int row = mt * 16 + n;  // position within the tile
         if (row < count) {
             const int position = first + row;
@@ -201,6 +234,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 }
             }
         }
+    }
+}
+
+template <bool GATE_UP, int R>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void a64_grouped_kernel(
+    SegGateUpArgs gu, SegDownArgs dn) {
+    const SegmentList& seg = GATE_UP ? gu.seg : dn.seg;
+    const int s = blockIdx.y;
+    if (s >= *seg.total) return;
+    const int first = seg.first[s];
+    const int count = seg.count[s];
+    const aeon_a64_expert e = (GATE_UP ? gu.experts : dn.experts)[seg.expert[s]];
+
+    // Activation windows in LDS, fragment-major: [ring slot][token tile][step][lane] x 16 bytes,
+    // so a B operand is one conflict-free ds_read_b128 per lane. 64 KiB: two slots of a full
+    // window, or a deeper ring of smaller ones.
+    __shared__ half8_t xs[2 * kGroupedMT * 4 * 64];
+
+    const int live_tiles = (count + 15) >> 4;
+    if (live_tiles > 4) {
+        grouped_run<GATE_UP, R, 8, 1>(gu, dn, e, first, count, xs);
+    } else if (live_tiles > 2) {
+        grouped_run<GATE_UP, R, 4, 3>(gu, dn, e, first, count, xs);
+    } else if (live_tiles > 1) {
+        grouped_run<GATE_UP, R, 2, 3>(gu, dn, e, first, count, xs);
+    } else {
+        grouped_run<GATE_UP, R, 1, 3>(gu, dn, e, first, count, xs);
     }
 }
 
