@@ -350,11 +350,10 @@ __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegD
 //     wave fetches one fragment (16 tokens x 32 columns) and all four read them from LDS.
 // Per wave and group that leaves NM*R weight loads + 1 activation load.
 template <bool GATE_UP, int R, int D>
-__global__ __launch_bounds__(256) void a64_seg_wide_kernel(SegGateUpArgs gu, SegDownArgs dn) {
+__device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const SegDownArgs& dn, int s,
+                                              int row_block, half8_t (*xs)[4][64], u32x4_t* scale_lds) {
     constexpr int NM = GATE_UP ? 2 : 1;
     const SegmentList& seg = GATE_UP ? gu.seg : dn.seg;
-    const int s = blockIdx.y;
-    if (s >= *seg.total) return;
     const int first = seg.first[s];
     const int count = seg.count[s];
     const aeon_a64_expert e = (GATE_UP ? gu.experts : dn.experts)[seg.expert[s]];
@@ -363,7 +362,7 @@ __global__ __launch_bounds__(256) void a64_seg_wide_kernel(SegGateUpArgs gu, Seg
     const int wave = threadIdx.x >> 6;
     const int n = lane & 15;
     const int chunk = lane >> 4;
-    const int tile0 = (blockIdx.x * 4 + wave) * R;
+    const int tile0 = (row_block * 4 + wave) * R;
 
     const int K = GATE_UP ? gu.H : dn.I;
     const int groups = K / 128;
@@ -387,8 +386,6 @@ __global__ __launch_bounds__(256) void a64_seg_wide_kernel(SegGateUpArgs gu, Seg
     // this wave's share of a group's activations: MFMA step `wave` (columns 32*wave..+31)
     xrow += wave * 32;
 
-    __shared__ half8_t xs[2][4][64];
-    extern __shared__ u32x4_t scale_lds[];  // [wave][m][r][groups * 2] 16-byte units
     const int tile_u4 = groups * 2;         // 32 bytes of scales per group
     u32x4_t* my_scales = scale_lds + static_cast<size_t>(wave) * NM * R * tile_u4;
 #pragma unroll
@@ -419,15 +416,24 @@ __global__ __launch_bounds__(256) void a64_seg_wide_kernel(SegGateUpArgs gu, Seg
 #pragma unroll
     for (int d = 0; d < D; ++d) load_group(d, d < groups ? d : groups - 1);
     xs[0][wave][lane] = *reinterpret_cast<const AEON_GLOBAL half8_t*>(xrow);
+    // This wave's activation fragments of the next D groups wait in registers, fetched as far
+    // ahead as the weights: loads complete in issue order, so a fragment fetched only one group
+    // ahead would force every weight request older than it to have landed by the end of each
+    // step and cut the weight pipeline to a single step whatever D is.
+    half8_t xr[D];
+    auto load_x = [&](int g) {
+        return *reinterpret_cast<const AEON_GLOBAL half8_t*>(xrow + (g < groups ? g : groups - 1) * 128);
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d) xr[(d + 1) % D] = load_x(d + 1);
     __syncthreads();
 
-    // step g: fetch this wave's fragment of group g+1, read all four fragments of group g from
-    // LDS, multiply, then publish the fetched fragment into the other LDS buffer. One barrier
-    // per group: buffer (g+1)&1 was last read in step g-1, before that step's barrier.
+    // step g: read all four fragments of group g from LDS, multiply, publish this wave's
+    // fragment of group g+1 (fetched D steps ago) into the other LDS buffer, then request group
+    // g+D's weights and group g+1+D's fragment. One barrier per group: buffer (g+1)&1 was last
+    // read in step g-1, before that step's barrier.
     const u32x2_t* scale_rows = reinterpret_cast<const u32x2_t*>(my_scales) + chunk;
     auto step = [&](int d, int g, bool refill) {
-        const int gx = g + 1 < groups ? g + 1 : g;  // the last step refetches its own group, unused
-        const half8_t xnext = *reinterpret_cast<const AEON_GLOBAL half8_t*>(xrow + gx * 128);
         half8_t xf[4];
 #pragma unroll
         for (int st = 0; st < 4; ++st) xf[st] = xs[g & 1][st][lane];
@@ -439,8 +445,11 @@ __global__ __launch_bounds__(256) void a64_seg_wide_kernel(SegGateUpArgs gu, Seg
                 const u32x2_t sc = scale_rows[((m * R + r) * tile_u4 + g * 2) * 2];
                 scale_add(acc[m][r], mfma_group(wq[d][m][r], xf), sc);
             }
-        if (refill) load_group(d, g + D);
-        xs[(g + 1) & 1][wave][lane] = xnext;
+        xs[(g + 1) & 1][wave][lane] = xr[(d + 1) % D];
+        if (refill) {
+            load_group(d, g + D);
+            xr[(d + 1) % D] = load_x(g + 1 + D);
+        }
         __syncthreads();
     };
     int g0 = 0;
@@ -481,7 +490,14 @@ __global__ __launch_bounds__(256) void a64_seg_wide_kernel(SegGateUpArgs gu, Seg
     }
 }
 
-int g_seg_depth = 2;  // measurement override of the pipeline depth
+template <bool GATE_UP, int R, int D>
+__global__ __launch_bounds__(256) void a64_seg_wide_kernel(SegGateUpArgs gu, SegDownArgs dn) {
+    __shared__ half8_t xs[2][4][64];
+    extern __shared__ u32x4_t scale_lds[];  // [wave][m][r][groups * 2] 16-byte units
+    const SegmentList& seg = GATE_UP ? gu.seg : dn.seg;
+    if (static_cast<int>(blockIdx.y) >= *seg.total) return;
+    seg_wide_item<GATE_UP, R, D>(gu, dn, blockIdx.y, blockIdx.x, xs, scale_lds);
+}
 
 template <bool GATE_UP, int R, int D>
 static void launch_seg_rd(const SegGateUpArgs& gu, const SegDownArgs& dn, int tiles, int capacity,
@@ -503,12 +519,12 @@ static void launch_seg_rd(const SegGateUpArgs& gu, const SegDownArgs& dn, int ti
 
 template <bool GATE_UP, int R>
 static void launch_seg_r(const SegGateUpArgs& gu, const SegDownArgs& dn, int tiles, int capacity,
-                         int k_split, hipStream_t stream) {
-    if (g_seg_depth >= 4) {
+                         int k_split, int depth, hipStream_t stream) {
+    if (depth >= 4) {
         launch_seg_rd<GATE_UP, R, 4>(gu, dn, tiles, capacity, k_split, stream);
-    } else if (g_seg_depth == 3) {
+    } else if (depth == 3) {
         launch_seg_rd<GATE_UP, R, 3>(gu, dn, tiles, capacity, k_split, stream);
-    } else if (g_seg_depth == 2) {
+    } else if (depth == 2) {
         launch_seg_rd<GATE_UP, R, 2>(gu, dn, tiles, capacity, k_split, stream);
     } else {
         launch_seg_rd<GATE_UP, R, 1>(gu, dn, tiles, capacity, k_split, stream);
@@ -517,35 +533,35 @@ static void launch_seg_r(const SegGateUpArgs& gu, const SegDownArgs& dn, int til
 
 template <bool GATE_UP>
 static void launch_seg(const SegGateUpArgs& gu, const SegDownArgs& dn, int tiles, int capacity,
-                       int k_split, int row_tiles, hipStream_t stream) {
+                       int k_split, int row_tiles, int depth, hipStream_t stream) {
     const bool direct = (GATE_UP ? gu.seg.total : dn.seg.total) == nullptr;
     if (k_split == 0 && (direct || tiles % (4 * (row_tiles >= 4 ? 4 : row_tiles >= 2 ? 2 : 1)) != 0)) {
         k_split = 1;  // the wide form needs a segment list and whole workgroups of tiles
     }
     if (row_tiles >= 4 && tiles % 4 == 0) {
-        launch_seg_r<GATE_UP, 4>(gu, dn, tiles, capacity, k_split, stream);
+        launch_seg_r<GATE_UP, 4>(gu, dn, tiles, capacity, k_split, depth, stream);
     } else if (row_tiles >= 2 && tiles % 2 == 0) {
-        launch_seg_r<GATE_UP, 2>(gu, dn, tiles, capacity, k_split, stream);
+        launch_seg_r<GATE_UP, 2>(gu, dn, tiles, capacity, k_split, depth, stream);
     } else {
-        launch_seg_r<GATE_UP, 1>(gu, dn, tiles, capacity, k_split, stream);
+        launch_seg_r<GATE_UP, 1>(gu, dn, tiles, capacity, k_split, depth, stream);
     }
 }
 
-int launch_seg_gate_up(const SegGateUpArgs& a, int k_split, int row_tiles, hipStream_t stream) {
+int launch_seg_gate_up(const SegGateUpArgs& a, int k_split, int row_tiles, int depth, hipStream_t stream) {
     AEON_REQUIRE(a.H % 128 == 0 && a.I % 16 == 0 && a.x_stride % 8 == 0, AEON_ERR_INVALID_ARGUMENT,
                  "gate/up segments: need H%%128==0, I%%16==0 and an activation pitch that keeps "
                  "rows 16-byte aligned (H=%d I=%d pitch=%ld)", a.H, a.I, a.x_stride);
     if (a.seg.capacity <= 0) return AEON_OK;
-    launch_seg<true>(a, SegDownArgs{}, a.I / 16, a.seg.capacity, k_split, row_tiles, stream);
+    launch_seg<true>(a, SegDownArgs{}, a.I / 16, a.seg.capacity, k_split, row_tiles, depth, stream);
     AEON_LAUNCH_CHECK();
     return AEON_OK;
 }
 
-int launch_seg_down(const SegDownArgs& a, int k_split, int row_tiles, hipStream_t stream) {
+int launch_seg_down(const SegDownArgs& a, int k_split, int row_tiles, int depth, hipStream_t stream) {
     AEON_REQUIRE(a.I % 128 == 0 && a.H % 16 == 0, AEON_ERR_INVALID_ARGUMENT,
                  "down segments: need I%%128==0 and H%%16==0 (H=%d I=%d)", a.H, a.I);
     if (a.seg.capacity <= 0) return AEON_OK;
-    launch_seg<false>(SegGateUpArgs{}, a, a.H / 16, a.seg.capacity, k_split, row_tiles, stream);
+    launch_seg<false>(SegGateUpArgs{}, a, a.H / 16, a.seg.capacity, k_split, row_tiles, depth, stream);
     AEON_LAUNCH_CHECK();
     return AEON_OK;
 }
@@ -666,7 +682,7 @@ extern "C" int aeon_a64_expert_decode(const void* d_x, int tokens, const aeon_a6
         gu.seg.capacity = 1;
         gu.direct_expert = *expert;
         gu.direct_count = tokens;
-        if (int rc = launch_seg_gate_up(gu, 4, 1, s)) return rc;
+        if (int rc = launch_seg_gate_up(gu, 4, 1, 2, s)) return rc;
         SegDownArgs dn{};
         dn.hidden = static_cast<const uint16_t*>(d_hidden);
         dn.weight = d_route_weights;
@@ -676,7 +692,7 @@ extern "C" int aeon_a64_expert_decode(const void* d_x, int tokens, const aeon_a6
         dn.seg.capacity = 1;
         dn.direct_expert = *expert;
         dn.direct_count = tokens;
-        if (int rc = launch_seg_down(dn, 4, 1, s)) return rc;
+        if (int rc = launch_seg_down(dn, 4, 1, 2, s)) return rc;
     } else {
         GemvArgs g{};
         g.x = static_cast<const uint16_t*>(d_x);

@@ -46,10 +46,9 @@ struct SegDownArgs {
 
 // k_split: 1, 2 or 4 waves of a workgroup split K between them. row_tiles: 1, 2 or 4
 // consecutive 16-row tiles per workgroup share one read of the activations.
-int launch_seg_gate_up(const SegGateUpArgs& a, int k_split, int row_tiles, hipStream_t stream);
-int launch_seg_down(const SegDownArgs& a, int k_split, int row_tiles, hipStream_t stream);
+int launch_seg_gate_up(const SegGateUpArgs& a, int k_split, int row_tiles, int depth, hipStream_t stream);
+int launch_seg_down(const SegDownArgs& a, int k_split, int row_tiles, int depth, hipStream_t stream);
 
-extern int g_seg_depth;
 
 // Prefill form: position tiles of up to kGroupedTokens per expert, weights dequantised into
 // MFMA fragments and reused across the tile's token tiles.

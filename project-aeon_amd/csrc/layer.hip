@@ -148,8 +148,9 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     int split_down = live_bound * (layer->hidden / 16) >= 8192 ? 0 : 4;
     int rows_gate = split_gate == 0 ? 2 : 1;
     int rows_down = split_down == 0 ? 4 : 1;
-    if (const char* t = getenv("AEON_TUNE")) {  // "kg rg kd rd": measurement override
-        sscanf(t, "%d %d %d %d %d", &split_gate, &rows_gate, &split_down, &rows_down, &g_seg_depth);
+    int depth_gate = 3, depth_down = 3;
+    if (const char* t = getenv("AEON_TUNE")) {  // "kg rg kd rd dg dd": measurement override
+        sscanf(t, "%d %d %d %d %d %d", &split_gate, &rows_gate, &split_down, &rows_down, &depth_gate, &depth_down);
     }
 
     SegGateUpArgs gu{};
@@ -164,7 +165,7 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     gu.limit = layer->swiglu_limit;
     if (stage_mask & AEON_STAGE_GATE_UP) {
         if (int rc = grouped ? launch_grouped_gate_up(gu, s)
-                             : launch_seg_gate_up(gu, split_gate, rows_gate, s)) {
+                             : launch_seg_gate_up(gu, split_gate, rows_gate, depth_gate, s)) {
             return rc;
         }
     }
@@ -180,7 +181,7 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     dn.I = layer->intermediate;
     if (stage_mask & AEON_STAGE_DOWN) {
         if (int rc = grouped ? launch_grouped_down(dn, s)
-                             : launch_seg_down(dn, split_down, rows_down, s)) {
+                             : launch_seg_down(dn, split_down, rows_down, depth_down, s)) {
             return rc;
         }
     }
