@@ -110,6 +110,119 @@ def run_prefill(layer, moe, capi, synth, torch, np, H, I, E, K_TOP, SEED, steps,
     }
 
 
+def run_other_configs(pool, layer, moe, capi, synth, torch, np, H, I, E, K_TOP, LIMIT, SEED, wr, bias,
+                      B, steps):
+    """Configs 0, 1 and 4 of BASELINE.json. Configs 0/1 rotate through every resident expert
+    (5.8 GB) so no launch finds its weights in the 256 MB Infinity Cache."""
+    def timed(fn, reps):
+        """Mean time of one call. The calls are a few microseconds long, shorter than a launch
+        through Python, so `reps` of them (each on a different expert) are captured into one HIP
+        graph and the graph's replay is what is timed."""
+        fn(0)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(reps):
+                fn(i + 1)
+        graph.replay()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(3):
+            graph.replay()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / (3 * reps)
+
+    res = {}
+    reps = max(4 * steps, 64)
+    bm = matrix_bytes(I, H)
+    # config 0: one [7168 -> 2048] GEMV, one token
+    x1 = torch.from_numpy(synth.activations(SEED, 1, H, unit=7)).cuda()
+    y1 = torch.empty(1, I, dtype=torch.float16, device="cuda")
+    tab = pool.host_table
+
+    def gemv(i):
+        s = i % pool.slots
+        capi.call("aeon_a64_gemv", capi.vp(x1), H, C.c_void_p(int(tab[s, 0])),
+                  C.c_void_p(int(tab[s, 1])), capi.vp(y1), I, 1, I, H, moe.stream_ptr())
+
+    ms = timed(gemv, reps)
+    b0 = bm + H * 2 + I * 2
+    res["config0_gemv"] = {"us": round(ms * 1e3, 2), "algorithmic_bytes": b0,
+                           "achieved_gbps": round(b0 / (ms * 1e-3) / 1e9, 1),
+                           "frac_of_peak": round(b0 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+    # config 1: one routed expert, batch 1/4/8 (gate+up dual GEMV, SwiGLU, W2, router weight)
+    res["config1_one_expert"] = []
+    for tokens in (1, 4, 8):
+        x = torch.from_numpy(synth.activations(SEED, tokens, H, unit=11)).cuda()
+        w = torch.from_numpy(synth.route_weights(SEED, tokens)).cuda()
+        hidden = torch.empty(tokens, I, dtype=torch.float16, device="cuda")
+        contrib = torch.empty(tokens, H, dtype=torch.float32, device="cuda")
+        out = torch.empty(tokens, H, dtype=torch.float16, device="cuda")
+        structs = [pool.expert_struct(s) for s in range(pool.slots)]
+
+        def expert(i):
+            capi.call("aeon_a64_expert_decode", capi.vp(x), tokens, C.byref(structs[i % pool.slots]),
+                      capi.vp(w), capi.vp(hidden), capi.vp(contrib), None, capi.vp(out), H, I,
+                      C.c_float(LIMIT), 1, moe.stream_ptr())
+
+        ms = timed(expert, reps)
+        b1 = 3 * bm + tokens * H * 2 * 2
+        res["config1_one_expert"].append(
+            {"batch": tokens, "us": round(ms * 1e3, 2), "us_per_token": round(ms * 1e3 / tokens, 2),
+             "algorithmic_bytes": b1, "achieved_gbps": round(b1 / (ms * 1e-3) / 1e9, 1),
+             "frac_of_peak": round(b1 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+    # config 4: 4 stacked layers (independent seeded weights), batch B, hyper-connection mix of 4
+    # residual streams between layers
+    layers, mixes = [layer], []
+    for l in range(1, 4):
+        p = moe.ExpertPool(E + 1, H, I)
+        assert p.fill_synthetic(seed=SEED + 100 * l, first_expert_id=0) == 0
+        wr_l = torch.from_numpy(synth.router_weight(SEED + 100 * l, H, E)).cuda()
+        bias_l = torch.from_numpy(synth.router_bias(SEED + 100 * l, E)).cuda()
+        layers.append(moe.MoeLayer(p, E, K_TOP, True, LIMIT, wr_l, bias_l, score_kind=1))
+    rng = np.random.default_rng(SEED)
+    for l in range(4):
+        mixes.append(moe.HyperConnection(rng.standard_normal(24).astype(np.float32)))
+    stack = moe.LayerStack(layers, mixes)
+    residual = torch.from_numpy(np.stack([synth.activations(SEED, B, H, unit=50 + j)
+                                          for j in range(4)])).cuda()
+    # a step over an even number of layers ends in the buffer it started from, so every timed
+    # step starts from a fresh copy of the seeded streams (a 3.7 MB device copy inside the timing)
+    work = torch.empty_like(residual)
+    scratch = (torch.empty_like(residual), torch.empty(B, H, dtype=torch.float16, device="cuda"))
+    work.copy_(residual)
+    stack.step(work, scratch)
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    reps4 = max(steps // 2, 5)
+    a.record()
+    for _ in range(reps4):
+        work.copy_(residual)
+        r = stack.step(work, scratch)
+    b.record()
+    torch.cuda.synchronize()
+    ms = a.elapsed_time(b) / reps4
+    distinct = []
+    trace = []
+    work.copy_(residual)
+    r = stack.step(work, scratch, trace)
+    for entry in trace:
+        distinct.append(int(torch.unique(entry[2]).numel()))
+    be = 3 * bm
+    bytes4 = sum((d + 1) * be + H * E * 4 + B * H * 2 * 2 + B * K_TOP * 8 for d in distinct) + \
+        4 * 2 * 4 * B * H * 2
+    res["config4_stack"] = {"layers": 4, "batch": B, "ms_per_step": round(ms, 4),
+                            "us_per_token": round(ms * 1e3 / B, 3),
+                            "distinct_routed_experts_per_layer": distinct,
+                            "algorithmic_bytes": int(bytes4),
+                            "achieved_gbps": round(bytes4 / (ms * 1e-3) / 1e9, 1),
+                            "frac_of_peak": round(bytes4 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                            "finite": bool(torch.isfinite(r.float()).all())}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -121,6 +234,9 @@ def main():
     ap.add_argument("--cpu-tokens", type=int, default=4,
                     help="tokens of the batch the CPU oracle is timed on")
     ap.add_argument("--no-prefill", action="store_true", help="skip the config-3 prefill leg")
+    ap.add_argument("--all-configs", action="store_true",
+                    help="also time configs 0 (single GEMV), 1 (one expert, batch 1/4/8) and 4 "
+                         "(4 stacked layers with the hyper-connection mix) into `other_configs`")
     ap.add_argument("--sweep", action="store_true",
                     help="also report batch 1/8/32/64 in the `sweep` field")
     args = ap.parse_args()
@@ -237,6 +353,11 @@ def main():
     flat_layer = moe.MoeLayer(pool, E, K_TOP, True, LIMIT, wr, torch.zeros_like(bias), score_kind=1)
     flat = run_decode(B, args.steps, args.warmup, layer=flat_layer)
 
+    other = None
+    if args.all_configs:
+        other = run_other_configs(pool, layer, moe, capi, synth, torch, np, H, I, E, K_TOP, LIMIT,
+                                  SEED, wr, bias, B, args.steps)
+
     prefill = None
     if not args.no_prefill:
         prefill = run_prefill(layer, moe, capi, synth, torch, np, H, I, E, K_TOP, SEED, args.steps,
@@ -319,6 +440,8 @@ def main():
         "frac_of_peak": round(flat["step_gbps"] / HBM_PEAK_GBPS, 4),
         "gate_up_ms": round(flat["gate_up_ms"], 4), "gate_up_gbps": round(flat["gate_up_gbps"], 1),
         "down_ms": round(flat["down_ms"], 4), "down_gbps": round(flat["down_gbps"], 1)}
+    if other is not None:
+        result["other_configs"] = other
     if prefill is not None:
         result["prefill"] = prefill
     if sweep is not None:

@@ -30,6 +30,7 @@ extern "C" {
 #define AEON_ERR_LOGIC 2
 #define AEON_ERR_OUT_OF_RANGE 3
 #define AEON_ERR_HIP 4
+#define AEON_ERR_IO 5 /* file missing, truncated or malformed: std::runtime_error in the shims */
 
 const char* aeon_last_error(void);
 /* ABI revision of this header. */
@@ -306,6 +307,59 @@ int aeon_hc_post(const void* d_layer_out, long layer_out_stride, const void* d_r
                  long token_stride, long stream_stride, const float* d_post_mix,
                  const float* d_comb_mix, int mix_per_token, void* d_residual_out, int tokens,
                  int hidden, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * `.aeon` expert container -> HBM-resident experts in the wave64 packing (load time)
+ * ---------------------------------------------------------------------------------------- */
+
+/* The expert half of AeonModelLoader (src/infrastructure/artifact/aeon_loader.hpp:318-470,
+ * get_expert_location :145-160, get_expert_data :163-166): the index file is a 32-byte header
+ * {"AEON_EXPERTS" (12 bytes), u32 version, u32 layers, u32 experts_per_layer, u64 payload_bytes}
+ * followed by one {u64 offset, u64 length} entry per (layer, expert), layer-major
+ * (scripts/convert_safetensors_to_aeon.py:463-486); the experts file is mapped read-only.
+ * Rejected with AEON_ERR_IO, as the reference rejects them with std::runtime_error: missing or
+ * short files, a wrong magic, a version other than `expected_version`, an entry whose length is
+ * not payload_bytes or whose offset is not a multiple of `sector_size` or runs past the file. */
+typedef struct aeon_expert_catalog aeon_expert_catalog;
+int aeon_expert_catalog_open(const char* index_path, const char* experts_path,
+                             uint32_t expected_version, uint32_t sector_size,
+                             aeon_expert_catalog** out);
+void aeon_expert_catalog_close(aeon_expert_catalog* catalog);
+int aeon_expert_catalog_info(const aeon_expert_catalog* catalog, uint32_t* layers,
+                             uint32_t* experts_per_layer, uint64_t* payload_bytes,
+                             uint32_t* version);
+/* Host pointer to one expert's payload inside the mapping (AEON_ERR_OUT_OF_RANGE for an index
+ * outside the catalog). */
+int aeon_expert_catalog_payload(const aeon_expert_catalog* catalog, uint32_t layer,
+                                uint32_t expert, const void** payload, uint64_t* bytes);
+
+/* Byte offsets of the six sub-tensors inside one `.aeon` expert payload for an expert of shape
+ * (hidden, intermediate): [W1 packed | W1 scale | W2 packed | W2 scale | W3 packed | W3 scale],
+ * group-32 fp16 scales, no padding -- the order and sizes of
+ * src/backend/swizzled_w4a16/core/swizzled_expert_format.hpp:11-30 (AEON_W1_PACKED_OFFSET ...
+ * AEON_SWIZZLED_EXPERT_BYTES), which are this function at (4096, 2048). */
+typedef struct {
+    size_t w1_packed, w1_scale, w2_packed, w2_scale, w3_packed, w3_scale, total;
+} aeon_payload_layout;
+int aeon_payload_layout_for(int hidden, int intermediate, aeon_payload_layout* out);
+
+/* One resident expert slot in the wave64 packing: bytes per slot (a multiple of 4096) and the
+ * six device views of the slot at `d_slot` -- the counterpart of UnifiedVRAMExpertPool's slot
+ * views (src/backend/swizzled_w4a16/core/vram_expert_pool.hpp:22-82) with every expert
+ * resident. */
+size_t aeon_a64_slot_bytes(int hidden, int intermediate);
+int aeon_a64_slot_views(void* d_slot, int hidden, int intermediate, aeon_a64_expert* out);
+
+/* Loads experts [first, first+count) of `layer` into consecutive slots of `d_pool` (slot i at
+ * d_pool + i*aeon_a64_slot_bytes): payload bytes are copied from the mapping to a device staging
+ * buffer and re-swizzled there into the wave64 packing, copy and repack of neighbouring experts
+ * overlapped on two streams of the library's own. `h_table[i]` receives
+ * the views of slot i (host array; copy it to the device as the layer's expert table).
+ * Blocks until the pool is complete. `*mismatches` (nullable) = number of 128-column groups
+ * whose four group-32 scales were not bit-equal (the wave64 packing stores one; must be 0). */
+int aeon_resident_load_layer(const aeon_expert_catalog* catalog, uint32_t layer, uint32_t first,
+                             uint32_t count, int hidden, int intermediate, void* d_pool,
+                             size_t pool_bytes, aeon_a64_expert* h_table, long* mismatches);
 
 /* ------------------------------------------------------------------------------------------
  * Synthetic experts on the device (benchmarks and tests)

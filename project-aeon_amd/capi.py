@@ -7,7 +7,7 @@ import subprocess
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libaeon_mi355.so")
 
-OK, ERR_INVALID_ARGUMENT, ERR_LOGIC, ERR_OUT_OF_RANGE, ERR_HIP = 0, 1, 2, 3, 4
+OK, ERR_INVALID_ARGUMENT, ERR_LOGIC, ERR_OUT_OF_RANGE, ERR_HIP, ERR_IO = 0, 1, 2, 3, 4, 5
 
 
 class AeonLogicError(RuntimeError):
@@ -15,7 +15,7 @@ class AeonLogicError(RuntimeError):
 
 
 _EXC = {ERR_INVALID_ARGUMENT: ValueError, ERR_LOGIC: AeonLogicError,
-        ERR_OUT_OF_RANGE: IndexError, ERR_HIP: RuntimeError}
+        ERR_OUT_OF_RANGE: IndexError, ERR_HIP: RuntimeError, ERR_IO: OSError}
 
 
 class W13Table(C.Structure):
@@ -31,6 +31,11 @@ class A64Expert(C.Structure):
     _fields_ = [("w1_packed", C.c_void_p), ("w1_scale", C.c_void_p),
                 ("w3_packed", C.c_void_p), ("w3_scale", C.c_void_p),
                 ("w2_packed", C.c_void_p), ("w2_scale", C.c_void_p)]
+
+
+class PayloadLayout(C.Structure):
+    _fields_ = [(n, C.c_size_t) for n in ("w1_packed", "w1_scale", "w2_packed", "w2_scale",
+                                           "w3_packed", "w3_scale", "total")]
 
 
 def build(verbose=False):
@@ -50,12 +55,22 @@ def lib():
             raise RuntimeError(
                 "libaeon_mi355.so is not built: run __graft_entry__.build() (or make -C "
                 "project-aeon_amd/csrc); there is no fallback path")
+        # PyTorch ships its own copy of the HIP runtime under a different file name. If this
+        # library is loaded first, the process ends up with two runtimes (the system one bound
+        # here, PyTorch's bound to the tensors), and the one bound here finds no device. Loading
+        # PyTorch's first makes the loader reuse it for this library too.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         _lib = C.CDLL(LIB_PATH)
         _lib.aeon_last_error.restype = C.c_char_p
         _lib.aeon_a64_packed_bytes.restype = C.c_size_t
         _lib.aeon_a64_scale_bytes.restype = C.c_size_t
         _lib.aeon_moe_layer_workspace_bytes.restype = C.c_size_t
         _lib.aeon_router_logits_workspace_bytes.restype = C.c_size_t
+        _lib.aeon_a64_slot_bytes.restype = C.c_size_t
+        _lib.aeon_expert_catalog_close.restype = None
     return _lib
 
 

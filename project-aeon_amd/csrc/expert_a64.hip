@@ -277,8 +277,10 @@ __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegD
     };
 #pragma unroll
     for (int d = 0; d < D; ++d) {
-        const int j = d < mine ? d : mine - 1;  // a short wave reloads its last group, unused
-        load_group(d, wave + j * WK);
+        // a short wave reloads its last group, unused; a wave with no group at all (fewer groups
+        // than waves) reloads the matrix's last group so that every address stays inside it
+        const int j = d < mine ? d : mine - 1;
+        load_group(d, mine > 0 ? wave + j * WK : groups - 1);
     }
     int j0 = 0;
     for (; j0 + 2 * D <= mine; j0 += D) {
@@ -508,9 +510,9 @@ static void launch_seg_rd(const SegGateUpArgs& gu, const SegDownArgs& dn, int ti
         const size_t scale_bytes = static_cast<size_t>(4) * (GATE_UP ? 2 : 1) * R * (k_dim / 128) * 32;
         a64_seg_wide_kernel<GATE_UP, R, D>
             <<<dim3(tiles / (4 * R), capacity), 256, scale_bytes, stream>>>(gu, dn);
-    } else if (k_split >= 4) {
+    } else if (k_split >= 4 && (GATE_UP ? gu.H : dn.I) >= 4 * 128) {
         a64_seg_kernel<GATE_UP, R, 4, D><<<grid, 256, 0, stream>>>(gu, dn);
-    } else if (k_split == 2) {
+    } else if (k_split >= 2 && (GATE_UP ? gu.H : dn.I) >= 2 * 128) {
         a64_seg_kernel<GATE_UP, R, 2, D><<<grid, 128, 0, stream>>>(gu, dn);
     } else {
         a64_seg_kernel<GATE_UP, R, 1, D><<<grid, 64, 0, stream>>>(gu, dn);

@@ -144,14 +144,16 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
                            (draws < layer->experts ? draws : layer->experts);
     // Many live segments: the wide kernels (k_split 0: four waves per workgroup sharing the
     // activations through LDS, no K split). Few: split K four ways so the chip still fills.
-    int split_gate = live_bound * (layer->intermediate / 16) >= 8192 ? 0 : 4;
-    int split_down = live_bound * (layer->hidden / 16) >= 8192 ? 0 : 4;
-    int rows_gate = split_gate == 0 ? 2 : 1;
-    int rows_down = split_down == 0 ? 4 : 1;
-    int depth_gate = 3, depth_down = 3;
-    if (const char* t = getenv("AEON_TUNE")) {  // "kg rg kd rd dg dd": measurement override
-        sscanf(t, "%d %d %d %d %d %d", &split_gate, &rows_gate, &split_down, &rows_down, &depth_gate, &depth_down);
-    }
+    const int split_gate = live_bound * (layer->intermediate / 16) >= 8192 ? 0 : 4;
+    const int split_down = live_bound * (layer->hidden / 16) >= 4000 ? 0 : 4;
+    // Wide form: 64 gate/up rows or 128 down rows per workgroup and four (three) K groups of
+    // weights in flight per wave measured best at batch 64 on both a concentrated and a spread
+    // routing; more rows per workgroup save activation reads but leave fewer workgroups to
+    // balance over the CUs.
+    const int rows_gate = 1;
+    const int rows_down = split_down == 0 ? (live_bound >= 32 ? 2 : 1) : 1;
+    const int depth_gate = split_gate == 0 ? 4 : 2;
+    const int depth_down = split_down == 0 ? 3 : 2;
 
     SegGateUpArgs gu{};
     gu.x = static_cast<const uint16_t*>(d_x);

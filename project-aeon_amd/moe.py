@@ -39,21 +39,37 @@ class ExpertPool:
         self.sb13 = lib.aeon_a64_scale_bytes(intermediate, hidden)
         self.pb2 = lib.aeon_a64_packed_bytes(hidden, intermediate)
         self.sb2 = lib.aeon_a64_scale_bytes(hidden, intermediate)
-        offs, at = [], 0
-        for b in (self.pb13, self.sb13, self.pb13, self.sb13, self.pb2, self.sb2):
-            offs.append(at)
-            at += (b + 255) // 256 * 256
-        self.offsets = offs
-        self.slot_bytes = (at + 4095) // 4096 * 4096
+        self.slot_bytes = lib.aeon_a64_slot_bytes(hidden, intermediate)
         self.payload_bytes = 2 * (self.pb13 + self.sb13) + self.pb2 + self.sb2
         self.buffer = torch.empty(slots * self.slot_bytes, dtype=torch.uint8, device=device)
         base = self.buffer.data_ptr()
         table = np.empty((slots, 6), dtype=np.int64)
+        view = capi.A64Expert()
         for s in range(slots):
-            for j in range(6):
-                table[s, j] = base + s * self.slot_bytes + offs[j]
+            capi.call("aeon_a64_slot_views", C.c_void_p(base + s * self.slot_bytes), hidden,
+                      intermediate, C.byref(view))
+            table[s] = [view.w1_packed, view.w1_scale, view.w3_packed, view.w3_scale,
+                        view.w2_packed, view.w2_scale]
         self.host_table = table
+        self.offsets = [int(v) - base for v in table[0]]  # of the six sub-tensors inside a slot
         self.table = torch.from_numpy(table).to(device)
+
+    def load_catalog(self, catalog, layer, first=0, count=None, first_slot=0):
+        """Experts [first, first+count) of `layer` of an opened `.aeon` expert catalog -> slots
+        first_slot.. of this pool (payload -> device staging -> wave64 repack). Returns
+        the number of 128-groups with unequal group-32 scales (must be 0)."""
+        count = self.slots - first_slot if count is None else count
+        table = (capi.A64Expert * count)()
+        mismatches = C.c_long(0)
+        capi.call("aeon_resident_load_layer", catalog, layer, first, count, self.H, self.I,
+                  C.c_void_p(self.buffer.data_ptr() + first_slot * self.slot_bytes),
+                  C.c_size_t((self.slots - first_slot) * self.slot_bytes), table,
+                  C.byref(mismatches))
+        for i in range(count):
+            got = [table[i].w1_packed, table[i].w1_scale, table[i].w3_packed, table[i].w3_scale,
+                   table[i].w2_packed, table[i].w2_scale]
+            assert got == [int(v) for v in self.host_table[first_slot + i]]
+        return mismatches.value
 
     def expert_struct(self, slot):
         return capi.A64Expert(*[int(v) for v in self.host_table[slot]])

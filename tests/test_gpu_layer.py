@@ -190,6 +190,28 @@ def test_config2_moe_layer_decode_reduced_experts(orc, B):
     assert np.array_equal(out2.cpu().numpy(), out)
 
 
+@pytest.mark.parametrize("H,I,B", [(256, 128, 3), (256, 384, 5), (768, 256, 17), (256, 128, 70)])
+def test_layer_on_minimal_shapes(orc, H, I, B):
+    """Shapes with fewer 128-column groups than a workgroup has K-split waves (a wave with no
+    group of its own must not fetch anything outside the matrix), odd group counts for the
+    pipeline tails, and a batch just over the grouped path's threshold on a one-group K."""
+    torch, h, capi, moe, synth = _setup()
+    E, k, limit = 5, 2, 7.0
+    pool = moe.ExpertPool(E + 1, H, I)
+    assert pool.fill_synthetic(seed=21, first_expert_id=0) == 0
+    wr, bias = synth.router_weight(21, H, E), synth.router_bias(21, E)
+    layer = moe.MoeLayer(pool, E, k, True, limit, h.to_dev(wr), h.to_dev(bias), score_kind=1)
+    x = synth.activations(21, B, H, unit=B)
+    d_x = h.dev_half(x)
+    out, ids, w = layer.decode(d_x)
+    torch.cuda.synchronize()
+    ids, w, out = ids.cpu().numpy(), w.cpu().numpy(), out.cpu().numpy()
+    experts = {int(e): h.Expert(21, int(e), H, I) for e in np.unique(ids)}
+    shared = h.Expert(21, E, H, I)
+    want = _oracle_layer(orc, h, experts, x, ids, w, shared, limit)
+    assert np.abs(out - want).max() <= 6e-3 * np.abs(want).max()
+
+
 def test_prefill_grouped_small_full_oracle(orc):
     """The grouped path end to end on a shape small enough for the oracle to cover every token:
     ragged experts (empty, a few tokens, more than one 128-position tile), top-4 of 16, shared
