@@ -282,6 +282,20 @@ const float* aeon_moe_layer_logits(const aeon_moe_layer* layer, int tokens, void
  * Hyper-connection stream mix (hc_mult = 4)
  * ---------------------------------------------------------------------------------------- */
 
+/* hc_project_kernel launch, src/architecture/deepseek_v4/kernels/hc_sinkhorn.hpp:22-90 (call sites
+ * layer/v4_layer_body_attention.hpp:101-104,127-132): the per-token dynamic mixes,
+ * mixes[t][m] = rsqrt(mean(r_t^2) + rms_eps) * sum_k r_t[k] * fn[m][k] for m < 24, r_t the token's
+ * flattened 4 x hidden residual (element (t, j, h) at t*token_stride + j*stream_stride + h, fp32
+ * as in the reference or fp16), fn fp32 [24][4*hidden] with k = j*hidden + h. */
+int aeon_hc_project(const void* d_residual, int residual_is_f32, long token_stride,
+                    long stream_stride, const float* d_fn, float* d_mixes, int tokens, int hidden,
+                    float rms_eps, void* stream);
+/* rmsnorm_wave32_kernel / rmsnorm_unit_wave32_kernel, src/platform/ops/rmsnorm.hpp:35-105 (the FFN
+ * norm site, v4_layer_body_attention.hpp:113-115): out[t][i] = half(x[t][i] *
+ * rsqrt(mean(x[t]^2) + eps) * weight[i]); fp16 in, out and weight, fp32 arithmetic;
+ * d_weight NULL = the weightless form. Row pitches in elements. */
+int aeon_rmsnorm(const void* d_x, long x_stride, const void* d_weight, void* d_out,
+                 long out_stride, int tokens, int dim, float eps, void* stream);
 /* hc_sinkhorn_normalize_kernel launch, src/architecture/deepseek_v4/kernels/
  * hc_sinkhorn.hpp:151-255: mixes [tokens][24] -> pre [tokens][4] = sigmoid(m*s0+b)+pre_eps,
  * post [tokens][4] = sigmoid(m*s1+b)*post_alpha, comb [tokens][16] (comb[i*4+j], i the

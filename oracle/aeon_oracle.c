@@ -526,6 +526,26 @@ void orc_hc_pre_combine(const double* residual, const double* pre_mix, int hc_mu
     }
 }
 
+void orc_hc_mixes(const double* residual, const double* fn, size_t mixes, size_t hc_hidden,
+                  double rms_eps, double* out) { /* :509-524 */
+    double sum_sq = 0.0;
+    for (size_t k = 0; k < hc_hidden; ++k) sum_sq += residual[k] * residual[k];
+    const double inv_rms = 1.0 / sqrt(sum_sq / (double)hc_hidden + rms_eps);
+    for (size_t m = 0; m < mixes; ++m) {
+        double dot = 0.0;
+        for (size_t k = 0; k < hc_hidden; ++k) dot += residual[k] * fn[m * hc_hidden + k];
+        out[m] = dot * inv_rms;
+    }
+}
+
+void orc_rmsnorm(const double* x, const double* weight, size_t dim, double eps, double* out) {
+    /* :146-169 */
+    double sum_sq = 0.0;
+    for (size_t i = 0; i < dim; ++i) sum_sq += x[i] * x[i];
+    const double inv_rms = 1.0 / sqrt(sum_sq / (double)dim + eps);
+    for (size_t i = 0; i < dim; ++i) out[i] = weight ? x[i] * inv_rms * weight[i] : x[i] * inv_rms;
+}
+
 void orc_hc_post(const double* layer_out, const double* residual, const double* post_mix,
                  const double* comb, int hc_mult, size_t hidden, int transpose_comb,
                  double* out) { /* :613-632 */

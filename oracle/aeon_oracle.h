@@ -134,6 +134,11 @@ void orc_hc_sinkhorn(const double* mixes, const double* hc_scale, const double* 
                      double* pre_mix, double* post_mix, double* comb);
 void orc_hc_pre_combine(const double* residual, const double* pre_mix, int hc_mult,
                         size_t hidden, double* out);
+/* hc_mixes, dsv4_oracle.hpp:509-524: residual [hc_hidden] flattened, fn [mixes][hc_hidden]. */
+void orc_hc_mixes(const double* residual, const double* fn, size_t mixes, size_t hc_hidden,
+                  double rms_eps, double* out);
+/* rmsnorm / rmsnorm_unit, dsv4_oracle.hpp:146-169: weight NULL = the weightless form. */
+void orc_rmsnorm(const double* x, const double* weight, size_t dim, double eps, double* out);
 void orc_hc_post(const double* layer_out, const double* residual, const double* post_mix,
                  const double* comb, int hc_mult, size_t hidden, int transpose_comb,
                  double* out);

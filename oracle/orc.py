@@ -319,6 +319,25 @@ def hc_pre_combine(residual, pre_mix, hidden):
     return out
 
 
+def hc_mixes(residual, fn, rms_eps=1e-6):
+    """residual [hc_mult*hidden] flattened, fn [mixes][hc_mult*hidden] -> mixes [mixes]."""
+    r = np.ascontiguousarray(residual, dtype=np.float64).ravel()
+    f = np.ascontiguousarray(fn, dtype=np.float64)
+    out = np.empty(f.shape[0])
+    lib().orc_hc_mixes(_ptr(r, C.c_double), _ptr(f, C.c_double), C.c_size_t(f.shape[0]),
+                       C.c_size_t(r.size), C.c_double(rms_eps), _ptr(out, C.c_double))
+    return out
+
+
+def rmsnorm(x, weight=None, eps=1e-6):
+    xv = np.ascontiguousarray(x, dtype=np.float64)
+    wv = None if weight is None else np.ascontiguousarray(weight, dtype=np.float64)
+    out = np.empty(xv.size)
+    lib().orc_rmsnorm(_ptr(xv, C.c_double), None if wv is None else _ptr(wv, C.c_double),
+                      C.c_size_t(xv.size), C.c_double(eps), _ptr(out, C.c_double))
+    return out
+
+
 def hc_post(layer_out, residual, post_mix, comb, hidden, transpose_comb=False):
     lo = np.ascontiguousarray(layer_out, dtype=np.float64)
     r = np.ascontiguousarray(residual, dtype=np.float64)

@@ -150,6 +150,21 @@ void ref_hc_pre_combine(const double* residual, const double* pre, int hc_mult, 
     std::memcpy(out, r.data(), hidden * sizeof(double));
 }
 
+void ref_hc_mixes(const double* residual, const double* fn, size_t mixes, size_t hc_hidden,
+                  double rms_eps, double* out) {
+    const std::vector<double> r = ref::hc_mixes(
+        std::vector<double>(residual, residual + hc_hidden), mixes,
+        [&](size_t m, size_t k) { return fn[m * hc_hidden + k]; }, hc_hidden, rms_eps);
+    std::memcpy(out, r.data(), mixes * sizeof(double));
+}
+
+void ref_rmsnorm(const double* x, const double* weight, size_t dim, double eps, double* out) {
+    const std::vector<double> xv(x, x + dim);
+    const std::vector<double> r = weight ? ref::rmsnorm(xv, std::vector<double>(weight, weight + dim), eps)
+                                         : ref::rmsnorm_unit(xv, eps);
+    std::memcpy(out, r.data(), dim * sizeof(double));
+}
+
 void ref_hc_post(const double* layer_out, const double* residual, const double* post,
                  const double* comb, int hc_mult, size_t hidden, int transpose, double* out) {
     const std::vector<double> r = ref::hc_post(

@@ -182,6 +182,137 @@ extern "C" int aeon_hc_pre_combine(const void* d_residual, int residual_is_f32, 
     return AEON_OK;
 }
 
+namespace aeon355 {
+
+// mixes[t][m] = rsqrt(mean(r^2) + eps) * sum_k r[k] * fn[m][k] over the token's flattened
+// hc_mult x hidden residual r. One workgroup per token reads the residual once and carries all
+// 24 dot products plus the sum of squares (the reference launches one block per (mix, token),
+// reading the residual 24 times); fn (24 rows of hc_mult*hidden floats) is shared by every
+// token and stays in L2. Thread partials are combined in a fixed order -- xor butterfly inside
+// a wave, then waves 0..3 in sequence -- so a run is reproducible bit for bit.
+constexpr int kHcMixes = kHc * (2 + kHc);
+
+template <bool RESIDUAL_F32>
+__global__ __launch_bounds__(256) void hc_project_kernel(
+    const void* __restrict__ residual, long token_stride, long stream_stride,
+    const float* __restrict__ fn, float* __restrict__ mixes, int hidden, float rms_eps) {
+    const int token = blockIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    float dot[kHcMixes];
+#pragma unroll
+    for (int m = 0; m < kHcMixes; ++m) dot[m] = 0.0f;
+    float sum_sq = 0.0f;
+    const size_t flat = static_cast<size_t>(kHc) * hidden;
+    for (int j = 0; j < kHc; ++j) {
+        for (int h = threadIdx.x * 4; h < hidden; h += 256 * 4) {
+            float r[4];
+            const size_t at = static_cast<size_t>(token) * token_stride + j * stream_stride + h;
+            if (RESIDUAL_F32) {
+                const float4 v = *reinterpret_cast<const float4*>(static_cast<const float*>(residual) + at);
+                r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w;
+            } else {
+                const uint2 v = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(residual) + at);
+                r[0] = half_bits_to_float(static_cast<uint16_t>(v.x & 0xFFFFu));
+                r[1] = half_bits_to_float(static_cast<uint16_t>(v.x >> 16));
+                r[2] = half_bits_to_float(static_cast<uint16_t>(v.y & 0xFFFFu));
+                r[3] = half_bits_to_float(static_cast<uint16_t>(v.y >> 16));
+            }
+            sum_sq += r[0] * r[0] + r[1] * r[1] + r[2] * r[2] + r[3] * r[3];
+            const float* f = fn + static_cast<size_t>(j) * hidden + h;
+#pragma unroll
+            for (int m = 0; m < kHcMixes; ++m) {
+                const float4 w = *reinterpret_cast<const float4*>(f + m * flat);
+                dot[m] += r[0] * w.x + r[1] * w.y + r[2] * w.z + r[3] * w.w;
+            }
+        }
+    }
+    __shared__ float partial[4][kHcMixes + 1];
+#pragma unroll
+    for (int m = 0; m < kHcMixes; ++m) {
+        const float v = wave_xor_sum(dot[m], 63);
+        if (lane == 0) partial[wave][m] = v;
+    }
+    const float sq = wave_xor_sum(sum_sq, 63);
+    if (lane == 0) partial[wave][kHcMixes] = sq;
+    __syncthreads();
+    if (threadIdx.x < kHcMixes) {
+        const float total_sq = ((partial[0][kHcMixes] + partial[1][kHcMixes]) + partial[2][kHcMixes]) +
+                               partial[3][kHcMixes];
+        const float total = ((partial[0][threadIdx.x] + partial[1][threadIdx.x]) + partial[2][threadIdx.x]) +
+                            partial[3][threadIdx.x];
+        mixes[static_cast<size_t>(token) * kHcMixes + threadIdx.x] =
+            total * rsqrtf(total_sq / static_cast<float>(flat) + rms_eps);
+    }
+}
+
+// out[t][i] = half(x[t][i] * rsqrt(mean(x[t]^2) + eps) * weight[i]); fp32 arithmetic, fp16 in and
+// out, fp16 weight (null = the weightless form). One workgroup per token; the sum of squares is
+// combined in the same fixed order as above.
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict__ x, long x_stride,
+                                                      const uint16_t* __restrict__ weight,
+                                                      uint16_t* __restrict__ out, long out_stride,
+                                                      int dim, float eps) {
+    const int token = blockIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const uint16_t* row = x + static_cast<size_t>(token) * x_stride;
+    float sum_sq = 0.0f;
+    for (int i = threadIdx.x; i < dim; i += 256) {
+        const float v = half_bits_to_float(row[i]);
+        sum_sq += v * v;
+    }
+    __shared__ float partial[4];
+    const float sq = wave_xor_sum(sum_sq, 63);
+    if (lane == 0) partial[wave] = sq;
+    __syncthreads();
+    const float inv_rms =
+        rsqrtf((((partial[0] + partial[1]) + partial[2]) + partial[3]) / static_cast<float>(dim) + eps);
+    uint16_t* dst = out + static_cast<size_t>(token) * out_stride;
+    for (int i = threadIdx.x; i < dim; i += 256) {
+        const float w = weight != nullptr ? half_bits_to_float(weight[i]) : 1.0f;
+        dst[i] = float_to_half_bits(half_bits_to_float(row[i]) * inv_rms * w);
+    }
+}
+
+}  // namespace aeon355
+
+using namespace aeon355;
+
+extern "C" int aeon_hc_project(const void* d_residual, int residual_is_f32, long token_stride,
+                               long stream_stride, const float* d_fn, float* d_mixes, int tokens,
+                               int hidden, float rms_eps, void* stream) {
+    const char* who = "aeon_hc_project";
+    AEON_REQUIRE(d_residual && d_fn && d_mixes, AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
+    AEON_REQUIRE(tokens >= 0 && hidden > 0 && hidden % 4 == 0 && token_stride % 4 == 0 &&
+                     stream_stride % 4 == 0,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: bad shape or pitch (hidden=%d)", who, hidden);
+    if (tokens == 0) return AEON_OK;
+    if (residual_is_f32) {
+        hc_project_kernel<true><<<tokens, 256, 0, as_stream(stream)>>>(
+            d_residual, token_stride, stream_stride, d_fn, d_mixes, hidden, rms_eps);
+    } else {
+        hc_project_kernel<false><<<tokens, 256, 0, as_stream(stream)>>>(
+            d_residual, token_stride, stream_stride, d_fn, d_mixes, hidden, rms_eps);
+    }
+    AEON_LAUNCH_CHECK();
+    return AEON_OK;
+}
+
+extern "C" int aeon_rmsnorm(const void* d_x, long x_stride, const void* d_weight, void* d_out,
+                            long out_stride, int tokens, int dim, float eps, void* stream) {
+    const char* who = "aeon_rmsnorm";
+    AEON_REQUIRE(d_x && d_out, AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
+    AEON_REQUIRE(tokens >= 0 && dim > 0 && x_stride >= dim && out_stride >= dim,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: bad shape or pitch (dim=%d)", who, dim);
+    if (tokens == 0) return AEON_OK;
+    rmsnorm_kernel<<<tokens, 256, 0, as_stream(stream)>>>(
+        static_cast<const uint16_t*>(d_x), x_stride, static_cast<const uint16_t*>(d_weight),
+        static_cast<uint16_t*>(d_out), out_stride, dim, eps);
+    AEON_LAUNCH_CHECK();
+    return AEON_OK;
+}
+
 extern "C" int aeon_hc_post(const void* d_layer_out, long layer_out_stride,
                             const void* d_residual_in, long token_stride, long stream_stride,
                             const float* d_post_mix, const float* d_comb_mix, int mix_per_token,

@@ -204,6 +204,55 @@ class HyperConnection:
         return residual_out
 
 
+class DynamicHyperConnection:
+    """The per-token form of the mix (the reference's layer body, v4_layer_body_attention.hpp:
+    99-115): mixes = project(residual) per token, Sinkhorn per token, pre-combine with the
+    token's own pre-mix, then the FFN RMSNorm; the post expansion uses the token's post/comb."""
+
+    def __init__(self, fn, hc_scale, hc_base, norm_weight=None, rms_eps=1e-6, pre_eps=1e-6,
+                 sinkhorn_eps=1e-6, post_alpha=2.0, iters=20, device="cuda"):
+        self.fn = torch.as_tensor(np.asarray(fn, dtype=np.float32)).contiguous().to(device)
+        self.scale = torch.as_tensor(np.asarray(hc_scale, dtype=np.float32)).to(device)
+        self.base = torch.as_tensor(np.asarray(hc_base, dtype=np.float32)).to(device)
+        self.norm_weight = None if norm_weight is None else \
+            torch.as_tensor(np.asarray(norm_weight, dtype=np.float16)).to(device)
+        self.eps = (rms_eps, pre_eps, sinkhorn_eps, post_alpha, iters)
+        self.mixes = self.pre = self.post = self.comb = None
+
+    def pre_mix(self, residual, x_pre, x_norm):
+        """residual fp16 [4][tokens][hidden] -> x_pre (pre-combined) and x_norm (normed), fp16
+        [tokens][hidden]; keeps the per-token mixes for post_mix."""
+        streams, tokens, hidden = residual.shape
+        rms_eps, pre_eps, sinkhorn_eps, post_alpha, iters = self.eps
+        dev = residual.device
+        self.mixes = torch.empty(tokens, 24, dtype=torch.float32, device=dev)
+        self.pre = torch.empty(tokens, 4, dtype=torch.float32, device=dev)
+        self.post = torch.empty(tokens, 4, dtype=torch.float32, device=dev)
+        self.comb = torch.empty(tokens, 16, dtype=torch.float32, device=dev)
+        capi.call("aeon_hc_project", capi.vp(residual), 0, C.c_long(residual.stride(1)),
+                  C.c_long(residual.stride(0)), capi.vp(self.fn), capi.vp(self.mixes), tokens, hidden,
+                  C.c_float(rms_eps), stream_ptr())
+        capi.call("aeon_hc_sinkhorn_normalize", capi.vp(self.mixes), capi.vp(self.scale),
+                  capi.vp(self.base), capi.vp(self.pre), capi.vp(self.post), capi.vp(self.comb),
+                  tokens, C.c_float(pre_eps), C.c_float(sinkhorn_eps), C.c_float(post_alpha), iters,
+                  stream_ptr())
+        capi.call("aeon_hc_pre_combine", capi.vp(residual), 0, C.c_long(residual.stride(1)),
+                  C.c_long(residual.stride(0)), capi.vp(self.pre), 4, capi.vp(x_pre),
+                  C.c_long(x_pre.stride(0)), tokens, hidden, stream_ptr())
+        capi.call("aeon_rmsnorm", capi.vp(x_pre), C.c_long(x_pre.stride(0)),
+                  capi.vp(self.norm_weight), capi.vp(x_norm), C.c_long(x_norm.stride(0)), tokens,
+                  hidden, C.c_float(rms_eps), stream_ptr())
+        return x_norm
+
+    def post_mix(self, layer_out, residual_in, residual_out):
+        streams, tokens, hidden = residual_in.shape
+        capi.call("aeon_hc_post", capi.vp(layer_out), C.c_long(layer_out.stride(0)),
+                  capi.vp(residual_in), C.c_long(residual_in.stride(1)),
+                  C.c_long(residual_in.stride(0)), capi.vp(self.post), capi.vp(self.comb), 1,
+                  capi.vp(residual_out), tokens, hidden, stream_ptr())
+        return residual_out
+
+
 class LayerStack:
     """BASELINE config 4: stacked MoE layers with the hyper-connection residual mix between them.
     Per layer: x = pre-combine(residual); y = MoE(x); residual = post-mix(y, residual)."""

@@ -107,6 +107,19 @@ def main():
                  ("comb", comb), ("res", res), ("layer_out", lo), ("pre_combine", xin), ("post_out", rout)):
         out["hc_" + k] = v
 
+    # dynamic mixes and RMSNorm (dsv4_oracle.hpp:509-524, :146-169)
+    mres, mfn = rng.normal(size=4 * 48), rng.normal(size=(24, 4 * 48))
+    mout = np.empty(24)
+    ref.ref_hc_mixes(P(mres, C.c_double), P(mfn, C.c_double), C.c_size_t(24), C.c_size_t(4 * 48),
+                     C.c_double(1e-6), P(mout, C.c_double))
+    nx, nw = rng.normal(size=80), rng.normal(size=80)
+    nout, nunit = np.empty(80), np.empty(80)
+    ref.ref_rmsnorm(P(nx, C.c_double), P(nw, C.c_double), C.c_size_t(80), C.c_double(1e-6), P(nout, C.c_double))
+    ref.ref_rmsnorm(P(nx, C.c_double), None, C.c_size_t(80), C.c_double(1e-6), P(nunit, C.c_double))
+    for k, v in (("mix_res", mres), ("mix_fn", mfn), ("mix_out", mout), ("norm_x", nx), ("norm_w", nw),
+                 ("norm_out", nout), ("norm_unit", nunit)):
+        out["dyn_" + k] = v
+
     path = os.path.join(ROOT, "tests", "golden", "ref_vectors.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path), "bytes")

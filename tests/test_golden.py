@@ -65,3 +65,6 @@ def test_swiglu_router_hc(orc, gold):
     assert np.array_equal(comb, gold["hc_comb"])
     assert np.array_equal(orc.hc_pre_combine(gold["hc_res"], pre, 64), gold["hc_pre_combine"])
     assert np.array_equal(orc.hc_post(gold["hc_layer_out"], gold["hc_res"], post, comb, 64), gold["hc_post_out"])
+    assert np.array_equal(orc.hc_mixes(gold["dyn_mix_res"], gold["dyn_mix_fn"]), gold["dyn_mix_out"])
+    assert np.array_equal(orc.rmsnorm(gold["dyn_norm_x"], gold["dyn_norm_w"]), gold["dyn_norm_out"])
+    assert np.array_equal(orc.rmsnorm(gold["dyn_norm_x"]), gold["dyn_norm_unit"])

@@ -90,6 +90,71 @@ def test_pre_combine_and_post_against_oracle(orc):
         hc.post_mix(d_lo, d_res, d_res)
 
 
+@pytest.mark.parametrize("tokens,H", [(1, 256), (5, 1024), (64, 7168)])
+def test_dynamic_mix_projection_norm_and_post(orc, tokens, H):
+    """The per-token mix: projection (rms-scaled dots with 24 fn rows), per-token Sinkhorn,
+    pre-combine with the token's own pre-mix, RMSNorm (weighted and weightless), and the post
+    expansion with the token's post/comb -- each stage against the oracle fed the stage's own
+    device input."""
+    torch, h, capi, moe, synth = _setup()
+    rng = np.random.default_rng(tokens * 1000 + H)
+    res = (rng.standard_normal((4, tokens, H)) * 1.5).astype(np.float16)
+    fn = (rng.standard_normal((24, 4 * H)) * 0.05).astype(np.float32)
+    scale = rng.standard_normal(3).astype(np.float32)
+    base = rng.standard_normal(24).astype(np.float32)
+    weight = (1.0 + 0.1 * rng.standard_normal(H)).astype(np.float16)
+    hc = moe.DynamicHyperConnection(fn, scale, base, weight)
+    d_res = h.to_dev(res)
+    x_pre = torch.empty(tokens, H, dtype=torch.float16, device="cuda")
+    x_norm = torch.empty(tokens, H, dtype=torch.float16, device="cuda")
+    hc.pre_mix(d_res, x_pre, x_norm)
+    torch.cuda.synchronize()
+    mixes, pre = hc.mixes.cpu().numpy(), hc.pre.cpu().numpy()
+    post, comb = hc.post.cpu().numpy(), hc.comb.cpu().numpy()
+    check = range(tokens) if tokens <= 8 else (0, 17, tokens - 1)
+    for t in check:
+        flat = res[:, t, :].astype(np.float64).ravel()
+        want = orc.hc_mixes(flat, fn.astype(np.float64), 1e-6)
+        # fp32 accumulation of 4H products: a few ulps of the largest term, measured on the
+        # scale the dot products themselves have
+        assert np.abs(mixes[t] - want).max() <= 2e-5 * max(1.0, np.abs(want).max())
+        wp, wq, wc = orc.hc_sinkhorn(mixes[t].astype(np.float64), scale, base, 4)
+        assert np.abs(pre[t] - wp).max() <= 1e-5 and np.abs(post[t] - wq).max() <= 1e-5
+        assert np.abs(comb[t] - wc).max() <= 1e-5
+        want_x = orc.hc_pre_combine(res[:, t, :].astype(np.float64), pre[t].astype(np.float64), H)
+        got_x = x_pre[t].cpu().numpy()
+        assert np.abs(got_x - want_x).max() <= 2e-3 * np.abs(want_x).max()
+        want_n = orc.rmsnorm(got_x.astype(np.float64), weight.astype(np.float64), 1e-6)
+        assert h.rel_err(x_norm[t].cpu().numpy(), want_n) <= 2e-3
+    # the fp32 residual the reference keeps gives the same mixes as its fp16 rounding here
+    mixes32 = torch.empty(tokens, 24, dtype=torch.float32, device="cuda")
+    d_res32 = h.to_dev(res.astype(np.float32))
+    capi.call("aeon_hc_project", capi.vp(d_res32), 1, C.c_long(d_res32.stride(1)),
+              C.c_long(d_res32.stride(0)), capi.vp(hc.fn), capi.vp(mixes32), tokens, H,
+              C.c_float(1e-6), h.stream_ptr())
+    assert torch.equal(mixes32, hc.mixes)
+    # weightless norm
+    unit = torch.empty_like(x_norm)
+    capi.call("aeon_rmsnorm", capi.vp(x_pre), C.c_long(H), None, capi.vp(unit), C.c_long(H), tokens, H,
+              C.c_float(1e-6), h.stream_ptr())
+    t = check[-1] if not isinstance(check, range) else tokens - 1
+    want_u = orc.rmsnorm(x_pre[t].cpu().numpy().astype(np.float64), None, 1e-6)
+    assert h.rel_err(unit[t].cpu().numpy(), want_u) <= 2e-3
+    # post expansion with per-token post/comb
+    y = h.dev_half((rng.standard_normal((tokens, H)) * 2).astype(np.float16))
+    d_out = torch.empty_like(d_res)
+    hc.post_mix(y, d_res, d_out)
+    torch.cuda.synchronize()
+    for t in check:
+        want_r = orc.hc_post(y[t].cpu().numpy().astype(np.float64), res[:, t, :].astype(np.float64),
+                             post[t].astype(np.float64), comb[t].astype(np.float64), H)
+        assert np.abs(d_out[:, t, :].cpu().numpy() - want_r).max() <= 2e-3 * np.abs(want_r).max()
+    # reproducible bit for bit
+    first = hc.mixes.clone()
+    hc.pre_mix(d_res, x_pre, x_norm)
+    assert torch.equal(first, hc.mixes)
+
+
 @pytest.mark.parametrize("B,H,I,E", [(64, 1024, 512, 16), (4, 7168, 2048, 12)])
 def test_config4_stacked_layers(orc, B, H, I, E):
     """Four MoE layers with independent seeded weights and the HC mix between them. Each layer is

@@ -229,3 +229,24 @@ def test_hc_matches_reference(orc, ref):
         ref.ref_hc_post(P(lo, C.c_double), P(res, C.c_double), P(post, C.c_double),
                         P(comb, C.c_double), 4, C.c_size_t(hidden), tr, P(want, C.c_double))
         assert np.array_equal(orc.hc_post(lo, res, post, comb, hidden, bool(tr)), want)
+
+
+def test_hc_mixes_and_rmsnorm_match_reference(orc, ref):
+    """hc_mixes (dsv4_oracle.hpp:509-524) and rmsnorm / rmsnorm_unit (:146-169), bit for bit."""
+    rng = np.random.default_rng(11)
+    for hc_hidden, rows in ((4 * 96, 24), (4 * 33, 5)):
+        res = rng.normal(size=hc_hidden)
+        fn = rng.normal(size=(rows, hc_hidden))
+        for eps in (1e-6, 0.5):
+            want = np.empty(rows)
+            ref.ref_hc_mixes(P(res, C.c_double), P(fn, C.c_double), C.c_size_t(rows),
+                             C.c_size_t(hc_hidden), C.c_double(eps), P(want, C.c_double))
+            assert np.array_equal(orc.hc_mixes(res, fn, eps), want)
+    for dim in (1, 7, 640):
+        x, w = rng.normal(size=dim), rng.normal(size=dim)
+        want = np.empty(dim)
+        ref.ref_rmsnorm(P(x, C.c_double), P(w, C.c_double), C.c_size_t(dim), C.c_double(1e-6),
+                        P(want, C.c_double))
+        assert np.array_equal(orc.rmsnorm(x, w, 1e-6), want)
+        ref.ref_rmsnorm(P(x, C.c_double), None, C.c_size_t(dim), C.c_double(1e-3), P(want, C.c_double))
+        assert np.array_equal(orc.rmsnorm(x, None, 1e-3), want)
