@@ -93,21 +93,48 @@ __global__ __launch_bounds__(256) void permutation_scatter_kernel(PermutationArg
         }
         return;
     }
-    for (int base = 0; base < a.draws && position < end; base += 64) {
-        const int d = base + lane;
-        const bool mine = d < a.draws && a.ids[d] == e;
-        const unsigned long long mask = __ballot(mine);
-        if (mine) {
-            const int at = position + __popcll(mask & ((1ull << lane) - 1ull));
-            a.token_indices[at] = d / a.slots;
-            a.draw_indices[at] = d;
-            if (a.weights_by_position != nullptr) a.weights_by_position[at] = a.weights_by_draw[d];
+    // The scan is a chain of loads whose results decide nothing about the next address, so
+    // 32 rounds of ids are requested together: the wave pays one memory latency per 2048
+    // draws instead of one per 64.
+    constexpr int kRounds = 32;
+    // token = draw / slots without the emulated integer division (it dominated the scan): the
+    // product with ceil(2^32 / slots) is exact while draw * slots < 2^32, which the launcher
+    // checks before choosing this form.
+    const unsigned magic = a.slots_reciprocal;
+    for (int base = 0; base < a.draws && position < end; base += 64 * kRounds) {
+        int id[kRounds];
+        float weight[kRounds];
+#pragma unroll
+        for (int j = 0; j < kRounds; ++j) {
+            const int d = base + j * 64 + lane;
+            id[j] = d < a.draws ? a.ids[d] : -1;
+            // fetched with the ids, not inside the branch below: a load there would stall the
+            // wave for a memory latency in every round that places anything
+            weight[j] = d < a.draws && a.weights_by_draw != nullptr ? a.weights_by_draw[d] : 0.0f;
         }
-        position += __popcll(mask);
+#pragma unroll
+        for (int j = 0; j < kRounds; ++j) {
+            const int d = base + j * 64 + lane;
+            const bool mine = id[j] == e;
+            const unsigned long long mask = __ballot(mine);
+            if (mine) {
+                const int at = position + __popcll(mask & ((1ull << lane) - 1ull));
+                a.token_indices[at] = magic != 0 ? static_cast<int>(__umulhi(static_cast<unsigned>(d), magic))
+                                                 : d / a.slots;
+                a.draw_indices[at] = d;
+                if (a.weights_by_position != nullptr) a.weights_by_position[at] = weight[j];
+            }
+            position += __popcll(mask);
+        }
     }
 }
 
-int launch_permutation(const PermutationArgs& a, hipStream_t stream) {
+int launch_permutation(const PermutationArgs& args, hipStream_t stream) {
+    PermutationArgs a = args;
+    a.slots_reciprocal = 0;
+    if (a.slots > 1 && static_cast<uint64_t>(a.draws) * a.slots < (1ull << 32)) {
+        a.slots_reciprocal = static_cast<unsigned>(((1ull << 32) + a.slots - 1) / a.slots);
+    }
     permutation_offsets_kernel<<<1, 1024, 0, stream>>>(a);
     AEON_LAUNCH_CHECK();
     const int lists = a.experts + (a.shared_tokens > 0 ? 1 : 0);

@@ -14,6 +14,7 @@ struct PermutationArgs {
     const int32_t* ids;  // [draws] expert of draw token*slots+slot
     int draws;
     int slots;
+    unsigned slots_reciprocal;  // filled by launch_permutation
     int experts;         // routed experts
     int shared_tokens;   // > 0: append one more list holding tokens 0..shared_tokens-1
     int32_t* offsets;    // [lists + 1]
