@@ -351,9 +351,15 @@ __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegD
 //   * the four waves share one copy of the segment's activation fragments: per group every
 //     wave fetches one fragment (16 tokens x 32 columns) and all four read them from LDS.
 // Per wave and group that leaves NM*R weight loads + 1 activation load.
-template <bool GATE_UP, int R, int D>
+// A segment of the wide form holds up to kWideSegTokens positions of one expert: MT = 1 or 2
+// token tiles of 16. Both tiles ride on one pass over the weights -- a word is unpacked once and
+// multiplied into each tile -- so an expert that drew 17..32 tokens (or the always-on expert's
+// long list) streams its weights once per 32 positions instead of once per 16.
+static_assert(kWideSegTokens == kWideMaxTiles * kSegTokens, "segment length of the wide form");
+
+template <bool GATE_UP, int R, int D, int MT>
 __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const SegDownArgs& dn, int s,
-                                              int row_block, half8_t (*xs)[4][64], u32x4_t* scale_lds) {
+                                              int row_block, half8_t* xs, u32x4_t* scale_lds) {
     constexpr int NM = GATE_UP ? 2 : 1;
     const SegmentList& seg = GATE_UP ? gu.seg : dn.seg;
     const int first = seg.first[s];
@@ -377,16 +383,21 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
         sm[NM - 1] = as_global<uint16_t>(e.w3_scale);
     }
 
-    const int position = first + (n < count ? n : count - 1);
-    const AEON_GLOBAL uint16_t* xrow;
-    if (GATE_UP) {
-        const long row = gu.row_index != nullptr ? gu.row_index[position] : position;
-        xrow = as_global<uint16_t>(gu.x) + row * gu.x_stride + chunk * 8;
-    } else {
-        xrow = as_global<uint16_t>(dn.hidden) + static_cast<size_t>(position) * dn.I + chunk * 8;
+    // this wave's share of a group's activations: MFMA step `wave` (columns 32*wave..+31) of
+    // every token tile; a padded token column repeats the segment's last live position
+    const AEON_GLOBAL uint16_t* xrow[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int token = mt * kSegTokens + n;
+        const int position = first + (token < count ? token : count - 1);
+        if (GATE_UP) {
+            const long row = gu.row_index != nullptr ? gu.row_index[position] : position;
+            xrow[mt] = as_global<uint16_t>(gu.x) + row * gu.x_stride + chunk * 8 + wave * 32;
+        } else {
+            xrow[mt] = as_global<uint16_t>(dn.hidden) + static_cast<size_t>(position) * dn.I + chunk * 8 +
+                       wave * 32;
+        }
     }
-    // this wave's share of a group's activations: MFMA step `wave` (columns 32*wave..+31)
-    xrow += wave * 32;
 
     const int tile_u4 = groups * 2;         // 32 bytes of scales per group
     u32x4_t* my_scales = scale_lds + static_cast<size_t>(wave) * NM * R * tile_u4;
@@ -399,11 +410,13 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
             for (int i = lane; i < tile_u4; i += 64) my_scales[(m * R + r) * tile_u4 + i] = src[i];
         }
 
-    float4_t acc[NM][R];
+    float4_t acc[NM][R][MT];
 #pragma unroll
     for (int m = 0; m < NM; ++m)
 #pragma unroll
-        for (int r = 0; r < R; ++r) acc[m][r] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc[m][r][mt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
     u32x4_t wq[D][NM][R];
     auto load_group = [&](int d, int g) {
@@ -415,19 +428,24 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
                 wq[d][m][r] = pm[m][t * 64 + lane];
             }
     };
+    // LDS image of a group's activations: [buffer][token tile][MFMA step][lane] x 16 bytes
+    auto slot = [&](int buffer, int mt, int st) { return xs + ((buffer * kWideMaxTiles + mt) * 4 + st) * 64 + lane; };
 #pragma unroll
     for (int d = 0; d < D; ++d) load_group(d, d < groups ? d : groups - 1);
-    xs[0][wave][lane] = *reinterpret_cast<const AEON_GLOBAL half8_t*>(xrow);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) *slot(0, mt, wave) = *reinterpret_cast<const AEON_GLOBAL half8_t*>(xrow[mt]);
     // This wave's activation fragments of the next D groups wait in registers, fetched as far
     // ahead as the weights: loads complete in issue order, so a fragment fetched only one group
     // ahead would force every weight request older than it to have landed by the end of each
     // step and cut the weight pipeline to a single step whatever D is.
-    half8_t xr[D];
-    auto load_x = [&](int g) {
-        return *reinterpret_cast<const AEON_GLOBAL half8_t*>(xrow + (g < groups ? g : groups - 1) * 128);
+    half8_t xr[D][MT];
+    auto load_x = [&](int g, int mt) {
+        return *reinterpret_cast<const AEON_GLOBAL half8_t*>(xrow[mt] + (g < groups ? g : groups - 1) * 128);
     };
 #pragma unroll
-    for (int d = 0; d < D; ++d) xr[(d + 1) % D] = load_x(d + 1);
+    for (int d = 0; d < D; ++d)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) xr[(d + 1) % D][mt] = load_x(d + 1, mt);
     __syncthreads();
 
     // step g: read all four fragments of group g from LDS, multiply, publish this wave's
@@ -436,21 +454,39 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
     // read in step g-1, before that step's barrier.
     const u32x2_t* scale_rows = reinterpret_cast<const u32x2_t*>(my_scales) + chunk;
     auto step = [&](int d, int g, bool refill) {
-        half8_t xf[4];
+        half8_t xf[MT][4];
 #pragma unroll
-        for (int st = 0; st < 4; ++st) xf[st] = xs[g & 1][st][lane];
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int st = 0; st < 4; ++st) xf[mt][st] = *slot(g & 1, mt, st);
 #pragma unroll
         for (int m = 0; m < NM; ++m)
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 // scales of (tile, group): 16 rows x 2 bytes; this lane's rows are 4*chunk..+3
                 const u32x2_t sc = scale_rows[((m * R + r) * tile_u4 + g * 2) * 2];
-                scale_add(acc[m][r], mfma_group(wq[d][m][r], xf), sc);
+                if (MT == 1) {
+                    scale_add(acc[m][r][0], mfma_group(wq[d][m][r], xf[0]), sc);
+                } else {
+                    half8_t a[4];
+#pragma unroll
+                    for (int st = 0; st < 4; ++st) a[st] = unpack8_vec(wq[d][m][r][st]);
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) {
+                        float4_t t = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                        for (int st = 0; st < 4; ++st)
+                            t = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[st], xf[mt][st], t, 0, 0, 0);
+                        scale_add(acc[m][r][mt], t, sc);
+                    }
+                }
             }
-        xs[(g + 1) & 1][wave][lane] = xr[(d + 1) % D];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) *slot((g + 1) & 1, mt, wave) = xr[(d + 1) % D][mt];
         if (refill) {
             load_group(d, g + D);
-            xr[(d + 1) % D] = load_x(g + 1 + D);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) xr[(d + 1) % D][mt] = load_x(g + 1 + D, mt);
         }
         __syncthreads();
     };
@@ -468,37 +504,51 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
         if (g0 + D + d < groups) step(d, g0 + D + d, false);
     }
 
-    if (n >= count) return;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int row0 = (tile0 + r) * 16 + chunk * 4;
-        if (GATE_UP) {
-            const float4_t& ga = acc[0][r];
-            const float4_t& up = acc[NM - 1][r];
-            uint2 packed;
-            packed.x = float_to_half_bits(clamped_swiglu(ga[0], up[0], gu.limit)) |
-                       (static_cast<uint32_t>(float_to_half_bits(
-                            clamped_swiglu(ga[1], up[1], gu.limit))) << 16);
-            packed.y = float_to_half_bits(clamped_swiglu(ga[2], up[2], gu.limit)) |
-                       (static_cast<uint32_t>(float_to_half_bits(
-                            clamped_swiglu(ga[3], up[3], gu.limit))) << 16);
-            *reinterpret_cast<uint2*>(gu.hidden + static_cast<size_t>(first + n) * gu.I + row0) = packed;
-        } else {
-            const float w = dn.weight[first + n];
-            const float4_t v = {w * acc[0][r][0], w * acc[0][r][1], w * acc[0][r][2], w * acc[0][r][3]};
-            const size_t out_row = dn.out_row != nullptr ? dn.out_row[first + n] : first + n;
-            *reinterpret_cast<float4_t*>(dn.contrib + out_row * dn.H + row0) = v;
+    for (int mt = 0; mt < MT; ++mt) {
+        const int token = mt * kSegTokens + n;
+        if (token >= count) continue;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int row0 = (tile0 + r) * 16 + chunk * 4;
+            if (GATE_UP) {
+                const float4_t& ga = acc[0][r][mt];
+                const float4_t& up = acc[NM - 1][r][mt];
+                uint2 packed;
+                packed.x = float_to_half_bits(clamped_swiglu(ga[0], up[0], gu.limit)) |
+                           (static_cast<uint32_t>(float_to_half_bits(
+                                clamped_swiglu(ga[1], up[1], gu.limit))) << 16);
+                packed.y = float_to_half_bits(clamped_swiglu(ga[2], up[2], gu.limit)) |
+                           (static_cast<uint32_t>(float_to_half_bits(
+                                clamped_swiglu(ga[3], up[3], gu.limit))) << 16);
+                *reinterpret_cast<uint2*>(gu.hidden + static_cast<size_t>(first + token) * gu.I + row0) = packed;
+            } else {
+                const float w = dn.weight[first + token];
+                const float4_t& a4 = acc[0][r][mt];
+                const float4_t v = {w * a4[0], w * a4[1], w * a4[2], w * a4[3]};
+                const size_t out_row = dn.out_row != nullptr ? dn.out_row[first + token] : first + token;
+                *reinterpret_cast<float4_t*>(dn.contrib + out_row * dn.H + row0) = v;
+            }
         }
     }
 }
 
+// Four waves per SIMD (128 registers a wave) is what hides the weight stream's latency for the
+// common one-tile segment; the rarer two-tile path is kept inside that budget by a shallower
+// prefetch ring rather than allowed to halve everyone's occupancy.
 template <bool GATE_UP, int R, int D>
-__global__ __launch_bounds__(256) void a64_seg_wide_kernel(SegGateUpArgs gu, SegDownArgs dn) {
-    __shared__ half8_t xs[2][4][64];
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void a64_seg_wide_kernel(
+    SegGateUpArgs gu, SegDownArgs dn) {
+    __shared__ half8_t xs[2 * kWideMaxTiles * 4 * 64];
     extern __shared__ u32x4_t scale_lds[];  // [wave][m][r][groups * 2] 16-byte units
     const SegmentList& seg = GATE_UP ? gu.seg : dn.seg;
-    if (static_cast<int>(blockIdx.y) >= *seg.total) return;
-    seg_wide_item<GATE_UP, R, D>(gu, dn, blockIdx.y, blockIdx.x, xs, scale_lds);
+    const int s = blockIdx.y;
+    if (s >= *seg.total) return;
+    if (seg.count[s] > kSegTokens) {
+        seg_wide_item<GATE_UP, R, (D > 2 ? 2 : D), 2>(gu, dn, s, blockIdx.x, xs, scale_lds);
+    } else {
+        seg_wide_item<GATE_UP, R, D, 1>(gu, dn, s, blockIdx.x, xs, scale_lds);
+    }
 }
 
 template <bool GATE_UP, int R, int D>

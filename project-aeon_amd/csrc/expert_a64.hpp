@@ -9,11 +9,15 @@ namespace aeon355 {
 // A segment is one expert with up to kSegTokens of its permuted positions: the unit of work of
 // the MFMA decode kernels (16 = the token dimension of v_mfma_f32_16x16x32_f16).
 constexpr int kSegTokens = 16;
+// The wide form of the kernels takes segments of up to two token tiles (count <= 32); the
+// K-split form takes one (count <= 16). The segment list must be cut accordingly.
+constexpr int kWideMaxTiles = 2;
+constexpr int kWideSegTokens = kWideMaxTiles * kSegTokens;
 
 struct SegmentList {
     const int* expert;  // [capacity] expert id of each segment
     const int* first;   // [capacity] first permuted position
-    const int* count;   // [capacity] 1..kSegTokens
+    const int* count;   // [capacity] 1..kSegTokens (1..kWideSegTokens for the wide form)
     const int* total;   // [1] number of live segments (device); null = "direct" mode: one
                         // segment, positions 0..direct_count-1 of direct_expert
     int capacity;       // grid bound: blocks past *total exit at once

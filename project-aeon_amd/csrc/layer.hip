@@ -129,15 +129,10 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     p.seg_first = w.seg_first;
     p.seg_count = w.seg_count;
     p.seg_total = w.seg_total;
-    // A decode batch walks 16-position segments with the weight-streaming kernels; a prefill
-    // chunk walks 128-position tiles with the grouped GEMM.
+    // A decode batch walks segments of one expert's positions with the weight-streaming kernels;
+    // a prefill chunk walks 128-position tiles with the grouped GEMM.
     const bool grouped = tokens > kDecodeMaxTokens;
     const int lists = layer->experts + (layer->has_shared ? 1 : 0);
-    p.seg_tokens = grouped ? kGroupedTokensPerTile : kSegTokens;
-    p.seg_capacity = grouped ? lists + w.positions / kGroupedTokensPerTile + 1 : w.seg_capacity;
-    if (stage_mask & AEON_STAGE_PERMUTATION) {
-        if (int rc = launch_permutation(p, s)) return rc;
-    }
 
     // Few live segments (a small batch) leave the chip idle unless K is also split.
     const int live_bound = (layer->has_shared ? (tokens + kSegTokens - 1) / kSegTokens : 0) +
@@ -154,6 +149,16 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     const int rows_down = split_down == 0 ? (live_bound >= 32 ? 2 : 1) : 1;
     const int depth_gate = split_gate == 0 ? 4 : 2;
     const int depth_down = split_down == 0 ? 3 : 2;
+    // When both launches take the wide form, a segment holds two token tiles, so an expert with
+    // 17..32 positions (and the always-on expert's list) streams its weights once, not twice.
+    const bool both_wide = split_gate == 0 && split_down == 0 &&
+                           (layer->intermediate / 16) % (4 * rows_gate) == 0 &&
+                           (layer->hidden / 16) % (4 * rows_down) == 0;
+    p.seg_tokens = grouped ? kGroupedTokensPerTile : both_wide ? kWideSegTokens : kSegTokens;
+    p.seg_capacity = grouped ? lists + w.positions / kGroupedTokensPerTile + 1 : w.seg_capacity;
+    if (stage_mask & AEON_STAGE_PERMUTATION) {
+        if (int rc = launch_permutation(p, s)) return rc;
+    }
 
     SegGateUpArgs gu{};
     gu.x = static_cast<const uint16_t*>(d_x);
