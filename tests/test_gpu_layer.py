@@ -212,6 +212,45 @@ def test_layer_on_minimal_shapes(orc, H, I, B):
     assert np.abs(out - want).max() <= 6e-3 * np.abs(want).max()
 
 
+def test_decode_segments_of_two_token_tiles(orc):
+    """A decode batch in which both launches take the wide form (many live experts) and single
+    experts hold 40, 20, 17 and 16 positions: segments of 32+8, 20, 17 and 16 positions, i.e. the
+    two-tile path with full, partial and barely-started second tiles next to one-tile segments.
+    The always-on expert's 64 tokens make two full two-tile segments."""
+    torch, h, capi, moe, synth = _setup()
+    H, I, E, k, T, limit = 1024, 2048, 80, 2, 64, 7.0
+    pool = moe.ExpertPool(E + 1, H, I)
+    assert pool.fill_synthetic(seed=13, first_expert_id=0) == 0
+    layer = moe.MoeLayer(pool, E, k, True, limit)
+    ids = np.empty((T, k), dtype=np.int32)
+    ids[:40, 0] = 3                       # 40 positions
+    ids[40:60, 0] = 7                     # 20
+    ids[60:, 0] = 11                      # 4
+    ids[:17, 1] = 5                       # 17
+    ids[17:33, 1] = 9                     # 16
+    ids[33:, 1] = 20 + np.arange(T - 33)  # one each: keeps the live-expert count high
+    w = synth.route_weights(13, T * k).reshape(T, k).astype(np.float32)
+    x = synth.activations(13, T, H)
+    d_x, d_ids, d_w = h.dev_half(x), h.to_dev(ids), h.to_dev(w)
+    out = layer.routed(d_x, d_ids, d_w).cpu().numpy()
+    check = [0, 16, 31, 32, 39, 40, 59, 60, 63]
+    needed = sorted(set(int(e) for t in check for e in ids[t]))
+    experts = {e: h.Expert(13, e, H, I) for e in needed}
+    shared = h.Expert(13, E, H, I)
+    want = _oracle_layer(orc, h, experts, x[check], ids[check], w[check], shared, limit)
+    assert np.abs(want).max() > 0.5
+    assert np.abs(out[check] - want).max() <= 6e-3 * np.abs(want).max()
+    # reversed token order: other positions share a segment, a token's own sums keep their order,
+    # so its output keeps its bits
+    rev = layer.routed(d_x.flip(0).contiguous(), d_ids.flip(0).contiguous(),
+                       d_w.flip(0).contiguous()).flip(0).cpu().numpy()
+    assert np.array_equal(rev, out)
+    # the K-split kernels a small batch takes sum K in four interleaved parts: same values to
+    # fp32 summation order
+    small = layer.routed(d_x[:8], d_ids[:8], d_w[:8]).cpu().numpy()
+    assert np.abs(small - out[:8]).max() <= 1e-3 * np.abs(out[:8]).max()
+
+
 def test_prefill_grouped_small_full_oracle(orc):
     """The grouped path end to end on a shape small enough for the oracle to cover every token:
     ragged experts (empty, a few tokens, more than one 128-position tile), top-4 of 16, shared
