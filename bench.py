@@ -42,12 +42,12 @@ def matrix_bytes(n, k):
     return n * k // 2 + n * (k // 128) * 2
 
 
-def measured_traffic(batch, experts):
+def measured_traffic(batch, experts, bias_scale=1.0):
     """HBM bytes per launch of the gate/up kernel from the committed rocprofv3 --pmc runs
     (FETCH_SIZE, WRITE_SIZE in KiB per dispatch, each scaled by what the same counter reads for a
     plain copy of known size), or None for a workload that was not profiled."""
     path = os.path.join(ROOT, "profiles", "traffic_config2_decode_b%d.json" % batch)
-    if experts != 256 or not os.path.exists(path):
+    if experts != 256 or bias_scale != 1.0 or not os.path.exists(path):
         return None
     t = json.load(open(path))
     return int(1024 * (t["fetch_size_kib_per_dispatch"] * t["fetch_scale"] +
@@ -237,6 +237,15 @@ def main():
     ap.add_argument("--all-configs", action="store_true",
                     help="also time configs 0 (single GEMV), 1 (one expert, batch 1/4/8) and 4 "
                          "(4 stacked layers with the hyper-connection mix) into `other_configs`")
+    ap.add_argument("--router-bias-scale", type=float, default=1.0,
+                    help="scale of the per-expert router bias in the headline leg (1 = BASELINE's "
+                         "N(0, 0.1); 0 = no bias, the spread routing)")
+    ap.add_argument("--no-unbiased", action="store_true",
+                    help="skip the second decode leg (router bias removed); a kernel profile of the "
+                         "run then holds the configured workload's launches only")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only copy 1 GiB device to device a few times and exit: the known-size kernel "
+                         "the FETCH_SIZE / WRITE_SIZE counters are scaled by")
     ap.add_argument("--sweep", action="store_true",
                     help="also report batch 1/8/32/64 in the `sweep` field")
     args = ap.parse_args()
@@ -254,6 +263,14 @@ def main():
         sys.exit("bench.py needs a GPU")
     capi.lib()
     torch.cuda.set_device(0)
+    if args.calibrate_copy:
+        src = torch.full((1 << 28,), 3, dtype=torch.int32, device="cuda")   # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes": int(src.numel() * 4), "copies": 4}))
+        return
     H, I, E, K_TOP, LIMIT, SEED = 7168, 2048, args.experts, 8, 7.0, 0
     B = args.batch
 
@@ -262,7 +279,7 @@ def main():
     bad = pool.fill_synthetic(seed=SEED, first_expert_id=0)
     assert bad == 0, "repack found group-32 scales that differ inside a 128-group"
     wr = torch.from_numpy(synth.router_weight(SEED, H, E)).cuda()
-    bias = torch.from_numpy(synth.router_bias(SEED, E)).cuda()
+    bias = torch.from_numpy(synth.router_bias(SEED, E)).cuda() * args.router_bias_scale
     layer = moe.MoeLayer(pool, E, K_TOP, True, LIMIT, wr, bias, score_kind=1)
     torch.cuda.synchronize()
     setup_s = time.time() - t_setup
@@ -350,8 +367,10 @@ def main():
     # less than the bias does, so the same high-bias experts win for most tokens and a batch of 64
     # touches ~95 distinct experts. The same step with the bias removed spreads over ~220 experts
     # (the figure a uniform choice gives) and is reported beside the headline.
-    flat_layer = moe.MoeLayer(pool, E, K_TOP, True, LIMIT, wr, torch.zeros_like(bias), score_kind=1)
-    flat = run_decode(B, args.steps, args.warmup, layer=flat_layer)
+    flat = None
+    if not args.no_unbiased:
+        flat_layer = moe.MoeLayer(pool, E, K_TOP, True, LIMIT, wr, torch.zeros_like(bias), score_kind=1)
+        flat = run_decode(B, args.steps, args.warmup, layer=flat_layer)
 
     other = None
     if args.all_configs:
@@ -414,32 +433,38 @@ def main():
         "config": {"workload": "config2: full MoE layer decode, batch %d, hidden 7168, "
                                "intermediate 2048, top-8 of %d experts + 1 shared, group-128 int4"
                                % (B, E),
+                   "router_bias_scale": args.router_bias_scale,
                    "batch": B, "experts": E, "resident_expert_bytes": pool.payload_bytes * (E + 1),
                    "distinct_routed_experts_per_step": round(main_run["distinct_experts_mean"], 1)},
         "step_hbm": {"algorithmic_bytes": int(main_run["step_bytes"]),
                      "achieved_gbps": round(main_run["step_gbps"], 1),
                      "frac_of_peak": round(main_run["step_gbps"] / HBM_PEAK_GBPS, 4)},
-        "roofline": {"kernel": "a64_seg_kernel<gate_up> (fused W1+W3 dual-GEMV + clamped SwiGLU)",
+        "roofline": {"kernel": "a64_seg_wide_kernel<gate_up> (fused W1+W3 dual-GEMV + clamped SwiGLU)",
                      "bound": "hbm",
                      "achieved": round(main_run["gate_up_gbps"], 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(main_run["gate_up_gbps"] / HBM_PEAK_GBPS, 4),
                      "avg_launch_ms": round(main_run["gate_up_ms"], 4),
                      "algorithmic_bytes": int(main_run["gate_up_bytes"]),
-                     "traffic": measured_traffic(B, E)},
+                     "traffic": measured_traffic(B, E, args.router_bias_scale)},
         "down_kernel": {"achieved_gbps": round(main_run["down_gbps"], 1),
                         "avg_launch_ms": round(main_run["down_ms"], 4),
                         "algorithmic_bytes": int(main_run["down_bytes"])},
         "cpu_baseline": cpu,
         "setup_s": round(setup_s, 1),
     }
-    result["decode_unbiased_router"] = {
-        "distinct_routed_experts_per_step": round(flat["distinct_experts_mean"], 1),
-        "ms_per_step": round(flat["ms_per_step"], 4), "us_per_token": round(flat["us_per_token"], 3),
-        "algorithmic_bytes": int(flat["step_bytes"]), "achieved_gbps": round(flat["step_gbps"], 1),
-        "frac_of_peak": round(flat["step_gbps"] / HBM_PEAK_GBPS, 4),
-        "gate_up_ms": round(flat["gate_up_ms"], 4), "gate_up_gbps": round(flat["gate_up_gbps"], 1),
-        "down_ms": round(flat["down_ms"], 4), "down_gbps": round(flat["down_gbps"], 1)}
+    if flat is not None:
+        result["decode_unbiased_router"] = {
+            "distinct_routed_experts_per_step": round(flat["distinct_experts_mean"], 1),
+            "ms_per_step": round(flat["ms_per_step"], 4),
+            "us_per_token": round(flat["us_per_token"], 3),
+            "algorithmic_bytes": int(flat["step_bytes"]),
+            "achieved_gbps": round(flat["step_gbps"], 1),
+            "frac_of_peak": round(flat["step_gbps"] / HBM_PEAK_GBPS, 4),
+            "gate_up_ms": round(flat["gate_up_ms"], 4),
+            "gate_up_gbps": round(flat["gate_up_gbps"], 1),
+            "gate_up_frac_of_peak": round(flat["gate_up_gbps"] / HBM_PEAK_GBPS, 4),
+            "down_ms": round(flat["down_ms"], 4), "down_gbps": round(flat["down_gbps"], 1)}
     if other is not None:
         result["other_configs"] = other
     if prefill is not None:
