@@ -231,7 +231,7 @@ def main():
     ap.add_argument("--batch", type=int, default=64, help="decode batch (1/8/32/64 in config 2)")
     ap.add_argument("--experts", type=int, default=256)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
-    ap.add_argument("--cpu-tokens", type=int, default=4,
+    ap.add_argument("--cpu-tokens", type=int, default=64,
                     help="tokens of the batch the CPU oracle is timed on")
     ap.add_argument("--no-prefill", action="store_true", help="skip the config-3 prefill leg")
     ap.add_argument("--all-configs", action="store_true",
@@ -386,14 +386,30 @@ def main():
     if not args.no_cpu:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         sys.path.insert(0, os.path.join(ROOT, "tests"))
-        import helpers
         import orc
         orc.lib()
         n_tok = min(args.cpu_tokens, B)
         x_host = main_run["x"][:n_tok].cpu().numpy()
         ids_host, w_host = main_run["ids"][:n_tok], main_run["w"][:n_tok]
         needed = sorted(set(int(e) for e in ids_host.ravel()) | {E})
-        experts = {e: helpers.Expert(SEED, e, H, I) for e in needed}   # untimed: input generation
+
+        # untimed: the oracle's inputs. The experts' `.aeon` payloads are regenerated by the device
+        # generator (bit-identical to the host generator, tests/test_gpu_layer.py) and copied back.
+        def payload(expert):
+            mats = []
+            for m, (n, k, cfg) in enumerate(((I, H, (4, 8)), (I, H, (4, 8)), (H, I, (8, 4)))):
+                p = torch.empty(n * k // 2, dtype=torch.uint8, device="cuda")
+                sc = torch.empty(n * k // 32, dtype=torch.int16, device="cuda")
+                capi.call("aeon_synth_matrix_swizzled", C.c_uint64(SEED), expert, m, n, k, cfg[0],
+                          cfg[1], capi.vp(p), capi.vp(sc), moe.stream_ptr())
+                mats.append((p.cpu().numpy().view(np.uint32), sc.cpu().numpy().view(np.uint16)))
+            return mats
+
+        def ffn(mats, x):
+            return orc.expert_ffn(mats[0], mats[1], mats[2], H, I, np.asarray(x, dtype=np.float64),
+                                  LIMIT, round_hidden=True)
+
+        experts = {e: payload(e) for e in needed}
         threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
         t0 = time.perf_counter()
         # expert-major, one expert decoded at a time, fp64, OpenMP over output rows
@@ -402,10 +418,10 @@ def main():
             if e == E:
                 continue
             rows, slots = np.nonzero(ids_host == e)
-            o = experts[e].ffn(x_host[rows], LIMIT, round_hidden=True)
+            o = ffn(experts[e], x_host[rows])
             for i, (t, s) in enumerate(zip(rows, slots)):
                 contrib[t, s] = float(w_host[t, s]) * o[i]
-        shared = experts[E].ffn(x_host, LIMIT, round_hidden=True)
+        shared = ffn(experts[E], x_host)
         ref_out = np.empty((n_tok, H))
         for t in range(n_tok):
             ref_out[t] = orc.moe_combine(contrib[t], shared[t].astype(np.float16).astype(np.float64))
