@@ -587,12 +587,11 @@ template <bool GATE_UP>
 static void launch_seg(const SegGateUpArgs& gu, const SegDownArgs& dn, int tiles, int capacity,
                        int k_split, int row_tiles, int depth, hipStream_t stream) {
     const bool direct = (GATE_UP ? gu.seg.total : dn.seg.total) == nullptr;
-    if (k_split == 0 && (direct || tiles % (4 * (row_tiles >= 4 ? 4 : row_tiles >= 2 ? 2 : 1)) != 0)) {
+    if (k_split == 0 && (direct || tiles % (4 * (row_tiles >= 2 ? 2 : 1)) != 0)) {
         k_split = 1;  // the wide form needs a segment list and whole workgroups of tiles
     }
-    if (row_tiles >= 4 && tiles % 4 == 0) {
-        launch_seg_r<GATE_UP, 4>(gu, dn, tiles, capacity, k_split, depth, stream);
-    } else if (row_tiles >= 2 && tiles % 2 == 0) {
+    // Two row tiles per wave is the most the 128-register budget of the wide form carries.
+    if (row_tiles >= 2 && tiles % 2 == 0) {
         launch_seg_r<GATE_UP, 2>(gu, dn, tiles, capacity, k_split, depth, stream);
     } else {
         launch_seg_r<GATE_UP, 1>(gu, dn, tiles, capacity, k_split, depth, stream);

@@ -48,8 +48,10 @@ struct SegDownArgs {
     int direct_count;
 };
 
-// k_split: 1, 2 or 4 waves of a workgroup split K between them. row_tiles: 1, 2 or 4
-// consecutive 16-row tiles per workgroup share one read of the activations.
+// k_split: 1, 2 or 4 waves of a workgroup split K between them; 0 = the wide form (four waves,
+// each with its own row tiles, activations shared through LDS). row_tiles: 1 or 2 consecutive
+// 16-row tiles per wave share one read of the activations. depth: K groups of weights in
+// flight per wave (1..4).
 int launch_seg_gate_up(const SegGateUpArgs& a, int k_split, int row_tiles, int depth, hipStream_t stream);
 int launch_seg_down(const SegDownArgs& a, int k_split, int row_tiles, int depth, hipStream_t stream);
 
