@@ -9,14 +9,14 @@
 namespace aeon355 {
 
 constexpr int kRouterTokenTile = 16;   // tokens per workgroup: the M of the fp32 MFMA
-constexpr int kRouterWaves = 8;        // waves per workgroup, each with its own slice of rows
+constexpr int kRouterWaves = 4;        // waves per workgroup, each with its own slice of rows
 constexpr int kRouterWaveRows = 112;   // rows of Wr per wave (7 MFMA passes of 16 rows)
 constexpr int kRouterChunkRows = kRouterWaves * kRouterWaveRows;  // rows per workgroup
 constexpr int kRouterMaxExperts = 1024;
 
 // partial[c][t][e] = sum over the rows h of chunk c of x[t][h] * Wr[h][e], on the fp32 matrix
 // cores (v_mfma_f32_16x16x4_f32: full fp32 operands and accumulate).
-// One workgroup = (chunk of 896 rows, 16 tokens, 64 experts). Each of its eight waves takes 112
+// One workgroup = (chunk of 448 rows, 16 tokens, 64 experts). Each of its four waves takes 112
 // rows; per 16 rows a lane reads 4 activations (8 bytes) and four float4 of Wr (row
 // 4*(l/16)+s, experts 4*(l%16)..+3 of the block -- 256 contiguous bytes per row), which feed
 // 16 MFMAs: component j of the float4 is the B operand of the tile holding experts 4n+j. The
@@ -135,14 +135,15 @@ __device__ __forceinline__ double router_score(double logit, int score_kind) {
     return sqrt(softplus);
 }
 
-// One workgroup of 256 threads per token. When `partial` is given the threads first sum the
-// token's logits over the chunks (ascending) into `logits`. Every thread then scores its experts
-// in fp64 and finds each one's rank under the total order (biased score descending, index
-// ascending) by comparing against all experts held in LDS: rank r < top_k is the r-th pick.
-// No serial scan and no cross-lane argmax, and the order -- ties to the lower index included --
-// is exactly the specification's.
-template <int kPerThread>
-__global__ __launch_bounds__(256) void router_topk_kernel(
+// One workgroup of 256 x kParts threads per token. When `partial` is given the first 256 threads
+// sum the token's logits over the chunks (ascending) into `logits` and score their experts in
+// fp64. Each expert's rank under the total order (biased score descending, index ascending) is
+// then counted against all experts held in LDS, the candidates split into kParts ranges whose
+// counts (integers, so the order of the adds does not matter) meet in LDS: rank r < top_k is the
+// r-th pick. No serial scan and no cross-lane argmax, and the order -- ties to the lower index
+// included -- is exactly the specification's.
+template <int kPerThread, int kParts>
+__global__ __launch_bounds__(256 * kParts) void router_topk_kernel(
     const float* __restrict__ partial, int chunks, int tokens, float* __restrict__ logits,
     const float* __restrict__ bias, const int64_t* __restrict__ hash_table,
     const int32_t* __restrict__ token_ids, float* __restrict__ topk_weights,
@@ -153,13 +154,14 @@ __global__ __launch_bounds__(256) void router_topk_kernel(
     __shared__ double score_lds[kPerThread * 256];
     __shared__ double picked_score[64];
     __shared__ int picked_id[64];
+    __shared__ int rank_lds[kPerThread * 256];
     float* out_row = logits + static_cast<size_t>(token) * experts;
-    double my_choice[kPerThread];
+    const int lane_expert = threadIdx.x % 256;
+    const int part = threadIdx.x / 256;
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j) {
-        const int e = threadIdx.x + 256 * j;
-        my_choice[j] = -1.0e300;
-        if (e < experts) {
+        const int e = lane_expert + 256 * j;
+        if (part == 0 && e < experts) {
             float acc;
             if (partial != nullptr) {
                 acc = 0.0f;
@@ -177,9 +179,9 @@ __global__ __launch_bounds__(256) void router_topk_kernel(
                 acc = out_row[e];
             }
             const double sc = router_score(static_cast<double>(acc), score_kind);
-            my_choice[j] = bias != nullptr ? sc + static_cast<double>(bias[e]) : sc;
             score_lds[e] = sc;
-            choice_lds[e] = my_choice[j];
+            choice_lds[e] = bias != nullptr ? sc + static_cast<double>(bias[e]) : sc;
+            rank_lds[e] = 0;
         }
     }
     __syncthreads();
@@ -193,20 +195,30 @@ __global__ __launch_bounds__(256) void router_topk_kernel(
             picked_score[threadIdx.x] = score_lds[e];
         }
     } else {
+        const int span = (experts + kParts - 1) / kParts;
+        const int first = part * span;
+        const int last = first + span < experts ? first + span : experts;
 #pragma unroll
         for (int j = 0; j < kPerThread; ++j) {
-            const int e = threadIdx.x + 256 * j;
+            const int e = lane_expert + 256 * j;
             if (e < experts) {
                 int rank = 0;
-                const double mine = my_choice[j];
-                for (int f = 0; f < experts; ++f) {
+                const double mine = choice_lds[e];
+                for (int f = first; f < last; ++f) {
                     const double other = choice_lds[f];
                     rank += (other > mine || (other == mine && f < e)) ? 1 : 0;
                 }
-                if (rank < top_k) {
-                    picked_id[rank] = e;
-                    picked_score[rank] = score_lds[e];
-                }
+                if (kParts > 1) atomicAdd(&rank_lds[e], rank);
+                else rank_lds[e] = rank;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < kPerThread; ++j) {
+            const int e = lane_expert + 256 * j;
+            if (part == 0 && e < experts && rank_lds[e] < top_k) {
+                picked_id[rank_lds[e]] = e;
+                picked_score[rank_lds[e]] = score_lds[e];
             }
         }
     }
@@ -245,11 +257,11 @@ int launch_router_topk(const float* partial, int chunks, float* logits, const fl
                        int32_t* topk_indices, int tokens, int experts, int top_k, float scaling,
                        int renormalize, int score_kind, hipStream_t stream) {
     if (experts <= 256) {
-        router_topk_kernel<1><<<tokens, 256, 0, stream>>>(
+        router_topk_kernel<1, 4><<<tokens, 1024, 0, stream>>>(
             partial, chunks, tokens, logits, bias, hash_table, token_ids, topk_weights,
             topk_indices, experts, top_k, scaling, renormalize, score_kind);
     } else {
-        router_topk_kernel<kRouterMaxExperts / 256><<<tokens, 256, 0, stream>>>(
+        router_topk_kernel<kRouterMaxExperts / 256, 1><<<tokens, 256, 0, stream>>>(
             partial, chunks, tokens, logits, bias, hash_table, token_ids, topk_weights,
             topk_indices, experts, top_k, scaling, renormalize, score_kind);
     }
