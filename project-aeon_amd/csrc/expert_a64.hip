@@ -542,7 +542,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     __shared__ half8_t xs[2 * kWideMaxTiles * 4 * 64];
     extern __shared__ u32x4_t scale_lds[];  // [wave][m][r][groups * 2] 16-byte units
     const SegmentList& seg = GATE_UP ? gu.seg : dn.seg;
-    const int s = blockIdx.y;
+    const int s = blockIdx.y;  // the list is ordered costliest first
     if (s >= *seg.total) return;
     if (seg.count[s] > kSegTokens) {
         seg_wide_item<GATE_UP, R, (D > 2 ? 2 : D), 2>(gu, dn, s, blockIdx.x, xs, scale_lds);

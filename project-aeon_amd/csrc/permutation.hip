@@ -61,17 +61,27 @@ __global__ __launch_bounds__(1024) void permutation_offsets_kernel(PermutationAr
     if (e == 0) a.offsets[lists] = total;
 
     if (a.seg_expert != nullptr) {
+        // Segments that are more than half full come first in the list, the short ones after
+        // them: the launches walk the list in order, so the costliest workgroups are dispatched
+        // first and the launch's tail is made of cheap ones.
         const int segments = (count + a.seg_tokens - 1) / a.seg_tokens;
-        const int seg_base = block_exclusive_scan(segments, wave_totals, &total);
+        const int last_count = count - (segments - 1) * a.seg_tokens;
+        const int light = segments > 0 && 2 * last_count <= a.seg_tokens ? 1 : 0;
+        const int heavy = segments - light;
+        int heavy_total = 0;
+        const int heavy_base = block_exclusive_scan(heavy, wave_totals, &total);
+        heavy_total = total;
+        const int light_base = block_exclusive_scan(light, wave_totals, &total);
+        const int all = heavy_total + total;
         for (int s = 0; s < segments; ++s) {
-            const int at = seg_base + s;
+            const int at = s < heavy ? heavy_base + s : heavy_total + light_base;
             if (at < a.seg_capacity) {
                 a.seg_expert[at] = e;
                 a.seg_first[at] = offset + s * a.seg_tokens;
                 a.seg_count[at] = min(a.seg_tokens, count - s * a.seg_tokens);
             }
         }
-        if (e == 0) *a.seg_total = min(total, a.seg_capacity);
+        if (e == 0) *a.seg_total = min(all, a.seg_capacity);
     }
 }
 
