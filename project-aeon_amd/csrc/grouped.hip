@@ -13,6 +13,8 @@
 //     tokens costs its weight stream and little else.
 // Weights are read once per (expert, position tile); tiles of one expert are adjacent in the
 // grid so their re-reads meet in L2 / Infinity Cache.
+#include <type_traits>
+
 #include "expert_a64.hpp"
 
 namespace aeon355 {
@@ -237,6 +239,213 @@ __device__ __forceinline__ void grouped_run(const SegGateUpArgs& gu, const SegDo
     }
 }
 
+// The body for a full window (eight token tiles), where arithmetic bounds the time. A K group is
+// 32 blocks; block (st, mt) is the NM*R MFMAs of MFMA step st on token tile mt. VALU work hides
+// behind the matrix pipe only when the same wave issues it right after an MFMA, so the group is
+// software-pipelined by hand, block by block:
+//   * the B fragments of a pair of blocks are read from LDS one pair early;
+//   * the weight fragments of MFMA step st+1 (for st = 3: step 0 of the next K group) are
+//     unpacked one fragment per two blocks, behind the MFMAs of step st;
+//   * a scheduling fence after every block keeps the compiler from regrouping any of it.
+// One K group of weights and activations is in flight while one is computed (two ring slots).
+template <bool GATE_UP, int R>
+__device__ __forceinline__ void grouped_run_full(const SegGateUpArgs& gu, const SegDownArgs& dn,
+                                                 const aeon_a64_expert& e, int first, int count,
+                                                 half8_t* xs_flat) {
+    constexpr int LIVE = kGroupedMT;
+    constexpr int NM = GATE_UP ? 2 : 1;
+    constexpr int kFrags = NM * R;
+    constexpr int kBufferStride = LIVE * 4 * 64;  // in 16-byte units
+    constexpr int kBlocks = 4 * LIVE;
+    static_assert(kFrags == 4, "one fragment is unpacked per two blocks");
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: LDS-DMA targets stay scalar
+    const int n = lane & 15;
+    const int chunk = lane >> 4;
+    const int tile0 = (blockIdx.x * 4 + wave) * R;
+
+    const int K = GATE_UP ? gu.H : dn.I;
+    const int groups = K / 128;
+    const AEON_GLOBAL char* pm[NM];
+    const AEON_GLOBAL char* sm[NM];
+    pm[0] = as_global<char>(GATE_UP ? e.w1_packed : e.w2_packed);
+    sm[0] = as_global<char>(GATE_UP ? e.w1_scale : e.w2_scale);
+    if (GATE_UP) {
+        pm[NM - 1] = as_global<char>(e.w3_packed);
+        sm[NM - 1] = as_global<char>(e.w3_scale);
+    }
+    uint32_t woff[R], soff[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const uint32_t t = static_cast<uint32_t>(tile0 + r) * groups;
+        woff[r] = (t * 64 + lane) * 16;
+        soff[r] = (t * 16 + n) * 2;
+    }
+    const AEON_GLOBAL char* xbase = as_global<char>(GATE_UP ? static_cast<const void*>(gu.x)
+                                                            : static_cast<const void*>(dn.hidden));
+    uint32_t xoff[LIVE];
+#pragma unroll
+    for (int j = 0; j < LIVE; ++j) {
+        const int row = j * 16 + n;
+        const int live_row = row < count ? row : count - 1;
+        const int position = first + live_row;
+        const int column = wave * 32 + chunk * 8;
+        if (GATE_UP) {
+            const long src_row = gu.row_index != nullptr ? gu.row_index[position] : position;
+            xoff[j] = static_cast<uint32_t>((src_row * gu.x_stride + column) * 2);
+        } else {
+            xoff[j] = static_cast<uint32_t>((static_cast<size_t>(position) * dn.I + column) * 2);
+        }
+    }
+
+    float4_t acc[NM][R][LIVE];
+#pragma unroll
+    for (int m = 0; m < NM; ++m)
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int mt = 0; mt < LIVE; ++mt) acc[m][r][mt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+    u32x4_t wq[2][NM][R];
+    uint16_t sc[2][NM][R];
+#define AEON_FULL_ISSUE(g_, stage_)                                                                 \
+    do {                                                                                            \
+        const int gi_ = (g_) < groups ? (g_) : groups - 1;                                          \
+        _Pragma("unroll") for (int j = 0; j < LIVE; ++j) {                                          \
+            __builtin_amdgcn_global_load_lds(                                                       \
+                (const AEON_GLOBAL void*)(xbase + (xoff[j] + static_cast<uint32_t>(gi_) * 256u)),   \
+                (__attribute__((address_space(3))) void*)(xs_flat + (stage_) * kBufferStride +      \
+                                                          (j * 4 + wave) * 64),                     \
+                16, 0, 0);                                                                          \
+        }                                                                                           \
+        _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                            \
+            _Pragma("unroll") for (int r = 0; r < R; ++r) {                                         \
+                wq[stage_][m][r] = *(const AEON_GLOBAL u32x4_t*)(                                   \
+                    pm[m] + (woff[r] + static_cast<uint32_t>(gi_) * 1024u));                        \
+                sc[stage_][m][r] = *(const AEON_GLOBAL uint16_t*)(                                  \
+                    sm[m] + (soff[r] + static_cast<uint32_t>(gi_) * 32u));                          \
+            }                                                                                       \
+        }                                                                                           \
+    } while (0)
+
+    auto scale_pair = [](uint16_t bits) {
+        union { uint16_t u; half_t h; } v;
+        v.u = bits;
+        return half2_t{v.h, v.h};
+    };
+    // B fragment of block i (token tile i % LIVE, MFMA step i / LIVE) of a ring slot.
+    auto fragment = [&](int slot, int i) {
+        return xs_flat[slot * kBufferStride + ((i % LIVE) * 4 + i / LIVE) * 64 + lane];
+    };
+
+    AEON_FULL_ISSUE(0, 0);
+    AEON_WAIT_VMCNT(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+
+    // weight fragments of the current MFMA step and of the next one: step st reads a[st % 2]
+    // and fills a[(st + 1) % 2]; four steps a group keep the parity the same in every group
+    half8_t a[2][NM][R];
+    half8_t b[4];
+#pragma unroll
+    for (int m = 0; m < NM; ++m)
+#pragma unroll
+        for (int r = 0; r < R; ++r) a[0][m][r] = scaled_fragment(wq[0][m][r][0], scale_pair(sc[0][m][r]));
+    b[0] = fragment(0, 0);
+    b[1] = fragment(0, 1);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // One K group out of ring slot s; group g+1 is requested into the other slot first.
+    // Blocks go in pairs. While LDS-DMA requests are outstanding the compiler waits for every
+    // LDS read at once, so the two reads of the next pair are placed behind the first MFMA of
+    // this pair -- behind the wait for this pair's own fragments -- and have the pair's eight
+    // MFMAs to land.
+    auto step = [&](int g, auto slot) {
+        constexpr int s = decltype(slot)::value;
+        constexpr int sn = 1 - s;
+        AEON_FULL_ISSUE(g + 1, sn);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < kBlocks; i += 2) {
+            const int st = i / LIVE, mt = i % LIVE;
+            if (i == 3 * LIVE) {
+                // this wave's requests for group g+1 were made a whole group's arithmetic ago;
+                // its weights are unpacked from here on
+                AEON_WAIT_VMCNT(0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            acc[0][0][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[st % 2][0][0], b[i % 4], acc[0][0][mt], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i + 2 < kBlocks) {
+                b[(i + 2) % 4] = fragment(s, i + 2);
+                b[(i + 3) % 4] = fragment(s, i + 3);
+            }
+#pragma unroll
+            for (int m = 0; m < NM; ++m)
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+                    if (m + r > 0)
+                        acc[m][r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[st % 2][m][r], b[i % 4],
+                                                                                acc[m][r][mt], 0, 0, 0);
+#pragma unroll
+            for (int m = 0; m < NM; ++m)
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+                    acc[m][r][mt + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[st % 2][m][r], b[(i + 1) % 4],
+                                                                                acc[m][r][mt + 1], 0, 0, 0);
+            {
+                const int f = mt / 2, m = f / R, r = f % R;
+                a[(st + 1) % 2][m][r] = st < 3 ? scaled_fragment(wq[s][m][r][st < 3 ? st + 1 : 0], scale_pair(sc[s][m][r]))
+                                      : scaled_fragment(wq[sn][m][r][0], scale_pair(sc[sn][m][r]));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // every wave's window of group g+1 has landed, and nobody reads slot s any more
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        b[0] = fragment(sn, 0);
+        b[1] = fragment(sn, 1);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    int g = 0;
+    for (; g + 2 <= groups; g += 2) {
+        step(g, std::integral_constant<int, 0>{});
+        step(g + 1, std::integral_constant<int, 1>{});
+    }
+    if (g < groups) step(g, std::integral_constant<int, 0>{});
+#undef AEON_FULL_ISSUE
+
+#pragma unroll
+    for (int mt = 0; mt < LIVE; ++mt) {
+        const int row = mt * 16 + n;  // position within the tile
+        if (row < count) {
+            const int position = first + row;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int row0 = (tile0 + r) * 16 + chunk * 4;
+                if (GATE_UP) {
+                    const float4_t& ga = acc[0][r][mt];
+                    const float4_t& up = acc[NM - 1][r][mt];
+                    uint2 packed;
+                    packed.x = float_to_half_bits(clamped_swiglu(ga[0], up[0], gu.limit)) |
+                               (static_cast<uint32_t>(float_to_half_bits(
+                                    clamped_swiglu(ga[1], up[1], gu.limit))) << 16);
+                    packed.y = float_to_half_bits(clamped_swiglu(ga[2], up[2], gu.limit)) |
+                               (static_cast<uint32_t>(float_to_half_bits(
+                                    clamped_swiglu(ga[3], up[3], gu.limit))) << 16);
+                    *reinterpret_cast<uint2*>(gu.hidden + static_cast<size_t>(position) * gu.I + row0) = packed;
+                } else {
+                    const float w = dn.weight[position];
+                    const float4_t& a4 = acc[0][r][mt];
+                    const float4_t v = {w * a4[0], w * a4[1], w * a4[2], w * a4[3]};
+                    const size_t out_row = dn.out_row != nullptr ? dn.out_row[position] : position;
+                    *reinterpret_cast<float4_t*>(dn.contrib + out_row * dn.H + row0) = v;
+                }
+            }
+        }
+    }
+}
+
 template <bool GATE_UP, int R>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void a64_grouped_kernel(
     SegGateUpArgs gu, SegDownArgs dn) {
@@ -254,7 +463,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     const int live_tiles = (count + 15) >> 4;
     if (live_tiles > 4) {
-        grouped_run<GATE_UP, R, 8, 1>(gu, dn, e, first, count, xs);
+        grouped_run_full<GATE_UP, R>(gu, dn, e, first, count, xs);
     } else if (live_tiles > 2) {
         grouped_run<GATE_UP, R, 4, 3>(gu, dn, e, first, count, xs);
     } else if (live_tiles > 1) {
