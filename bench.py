@@ -67,6 +67,42 @@ def settle(fn, torch, seconds=0.3):
         torch.cuda.synchronize()
 
 
+def calibrate_mfma(capi, torch):
+    """Sustained fp16 matrix-pipe rates of this GPU, for reading the prefill figure: the
+    library's register-resident MFMA loop (two waves per SIMD) with constant and with random
+    operands, and torch's fp16 matmul (the vendor GEMM) at 8192^3."""
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    wgs = cus * 2
+    sink = torch.empty(wgs * 256, dtype=torch.float32, device="cuda")
+    out = {"cus": cus, "mfma_peak_tflops": MFMA_F16_PEAK_TFLOPS}
+    for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
+        flop = C.c_double(0.0)
+
+        def launch(i=0):
+            capi.call("aeon_calibrate_mfma_f16", rnd, 40000, wgs, capi.vp(sink),
+                      C.c_size_t(sink.numel()), C.byref(flop), None)
+        settle(launch, torch, seconds=0.3)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(5):
+            launch()
+        b.record()
+        torch.cuda.synchronize()
+        out["mfma_loop_tflops_" + name] = round(flop.value * 5 / (a.elapsed_time(b) * 1e-3) / 1e12, 1)
+    n = 8192
+    x = torch.randn(n, n, device="cuda", dtype=torch.float16)
+    y = torch.randn(n, n, device="cuda", dtype=torch.float16)
+    settle(lambda i: torch.matmul(x, y), torch, seconds=0.3)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(20):
+        torch.matmul(x, y)
+    b.record()
+    torch.cuda.synchronize()
+    out["library_gemm_8192_tflops"] = round(2.0 * n ** 3 * 20 / (a.elapsed_time(b) * 1e-3) / 1e12, 1)
+    return out
+
+
 def run_prefill(layer, moe, capi, synth, torch, np, H, I, E, K_TOP, SEED, steps, warmup):
     """BASELINE config 3: 2048 tokens, top-8 of 256 experts with Zipf(1.1) popularity, through the
     permutation -> grouped gate+up GEMM + SwiGLU -> grouped W2 GEMM -> fixed-order reduce path.
@@ -260,6 +296,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only copy 1 GiB device to device a few times and exit: the known-size kernel "
                          "the FETCH_SIZE / WRITE_SIZE counters are scaled by")
+    ap.add_argument("--calibrate-mfma", action="store_true",
+                    help="only measure the sustained fp16 MFMA rate (register-resident loop with "
+                         "constant and with random operands) and a library fp16 GEMM, for context")
     ap.add_argument("--sweep", action="store_true",
                     help="also report batch 1/8/32/64 in the `sweep` field")
     args = ap.parse_args()
@@ -283,7 +322,21 @@ def main():
         for _ in range(4):
             dst.copy_(src)
         torch.cuda.synchronize()
-        print(json.dumps({"calibrate_copy_bytes": int(src.numel() * 4), "copies": 4}))
+        # the same copy timed with warm clocks: what a plain stream sustains on this GPU
+        settle(lambda i: dst.copy_(src), torch, seconds=0.3)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(20):
+            dst.copy_(src)
+        b.record()
+        torch.cuda.synchronize()
+        moved = 2.0 * src.numel() * 4 * 20
+        print(json.dumps({"calibrate_copy_bytes": int(src.numel() * 4), "copies": 4,
+                          "timed_copy_read_plus_write_gbps":
+                              round(moved / (a.elapsed_time(b) * 1e-3) / 1e9, 1)}))
+        return
+    if args.calibrate_mfma:
+        print(json.dumps(calibrate_mfma(capi, torch)))
         return
     H, I, E, K_TOP, LIMIT, SEED = 7168, 2048, args.experts, 8, 7.0, 0
     B = args.batch

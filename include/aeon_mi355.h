@@ -386,6 +386,19 @@ int aeon_resident_load_layer(const aeon_expert_catalog* catalog, uint32_t layer,
 int aeon_synth_matrix_swizzled(uint64_t seed, int expert, int matrix, int N, int K, int rpw,
                                int lpr, void* d_packed, void* d_scale, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Measurement aid (no counterpart in the reference)
+ * ---------------------------------------------------------------------------------------- */
+
+/* Launches `workgroups` workgroups of four waves that each run `iterations` rounds of 16
+ * independent v_mfma_f32_16x16x32_f16 out of registers, with constant (random_operands = 0) or
+ * pseudo-random fp16 operands, and writes one float per thread to d_sink (>= workgroups*256
+ * floats). *flop (host, optional) receives the FLOPs of the launch. Timed by the caller, it
+ * gives the matrix-pipe rate this GPU sustains at the clock its power limit allows for such
+ * data: the practical ceiling next to the published fp16 peak. */
+int aeon_calibrate_mfma_f16(int random_operands, int iterations, int workgroups, float* d_sink,
+                            size_t sink_floats, double* flop, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

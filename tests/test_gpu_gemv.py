@@ -242,3 +242,22 @@ def test_config1_one_expert_decode(orc, tokens, use_mfma):
     # of the peak (6e-3, tests/test_v4_expert_oracle.cpp:75-77)
     unrounded = e.ffn(x, limit, round_hidden=False) * w.astype(np.float64)[:, None]
     assert np.abs(out.cpu().numpy() - unrounded).max() <= 6e-3 * np.abs(unrounded).max()
+
+
+def test_mfma_calibration_loop_runs_and_counts_its_flops():
+    """The measurement aid: constant operands of 1.0 make every accumulator entry iterations*32,
+    so the sink is checkable in closed form; random operands only have to stay finite."""
+    torch, _, capi = _setup()
+    wgs, iters = 8, 50
+    sink = torch.zeros(wgs * 256, dtype=torch.float32, device="cuda")
+    flop = C.c_double(0.0)
+    capi.call("aeon_calibrate_mfma_f16", 0, iters, wgs, capi.vp(sink), C.c_size_t(sink.numel()),
+              C.byref(flop), None)
+    torch.cuda.synchronize()
+    assert flop.value == wgs * 4 * iters * 16 * 16384.0
+    # 16 tiles x 4 entries per lane, each the sum of `iters` MFMAs of 32 products of 1.0
+    assert torch.all(sink == 16 * 4 * iters * 32.0)
+    capi.call("aeon_calibrate_mfma_f16", 1, iters, wgs, capi.vp(sink), C.c_size_t(sink.numel()),
+              None, None)
+    torch.cuda.synchronize()
+    assert torch.isfinite(sink).all()
