@@ -40,16 +40,24 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int* wave_totals, int
     return result;
 }
 
+// A batch of at most this many draws is scattered by the workgroup that counts it (one launch
+// instead of two: a decode step is short enough for a launch to show).
+constexpr int kFusedScatterDraws = 1024;
+
+template <bool SCATTER>
 __global__ __launch_bounds__(1024) void permutation_offsets_kernel(PermutationArgs a) {
     __shared__ int histogram[kMaxPermutationExperts + 1];
     __shared__ int wave_totals[16];
     __shared__ int total;
+    __shared__ int draw_expert[SCATTER ? kFusedScatterDraws : 1];
     const int lists = a.experts + (a.shared_tokens > 0 ? 1 : 0);
     for (int e = threadIdx.x; e <= kMaxPermutationExperts; e += blockDim.x) histogram[e] = 0;
     __syncthreads();
     for (int d = threadIdx.x; d < a.draws; d += blockDim.x) {
         const int e = a.ids[d];
-        if (e >= 0 && e < a.experts) atomicAdd(&histogram[e], 1);
+        const bool valid = e >= 0 && e < a.experts;
+        if (valid) atomicAdd(&histogram[e], 1);
+        if (SCATTER) draw_expert[d] = valid ? e : -1;
     }
     if (threadIdx.x == 0 && a.shared_tokens > 0) histogram[a.experts] = a.shared_tokens;
     __syncthreads();
@@ -82,6 +90,48 @@ __global__ __launch_bounds__(1024) void permutation_offsets_kernel(PermutationAr
             }
         }
         if (e == 0) *a.seg_total = min(all, a.seg_capacity);
+    }
+
+    if (SCATTER) {
+        // Draw d goes to its list's offset plus the number of earlier draws of the same expert
+        // (ascending draw order inside a list). Wave w holds draws 64w..64w+63: the earlier
+        // waves' share comes from per-wave counts in LDS, the share of the lower lanes from a
+        // walk over the wave's own 64 draws.
+        __shared__ uint32_t wave_count_words[(kFusedScatterDraws / 64) * (kMaxPermutationExperts + 1) / 2 + 1];
+        unsigned short* wave_count = reinterpret_cast<unsigned short*>(wave_count_words);
+        const int lane = threadIdx.x & 63;
+        const int wave = threadIdx.x >> 6;
+        const int waves = (a.draws + 63) / 64;
+        for (int i = threadIdx.x; i < (waves * lists + 1) / 2; i += blockDim.x) wave_count_words[i] = 0;
+        __syncthreads();
+        if (e < lists) histogram[e] = offset;
+        const int d = threadIdx.x;
+        const int mine = d < a.draws ? draw_expert[d] : -1;
+        int rank = 0, later = 0;
+#pragma unroll 8
+        for (int l = 0; l < 64; ++l) {
+            const bool same = __builtin_amdgcn_readlane(mine, l) == mine;
+            rank += (l < lane && same) ? 1 : 0;
+            later += (l > lane && same) ? 1 : 0;
+        }
+        // the last lane of an expert in the wave knows the wave's count for it
+        if (mine >= 0 && later == 0) wave_count[wave * lists + mine] = static_cast<unsigned short>(rank + 1);
+        __syncthreads();
+        if (mine >= 0) {
+            for (int w = 0; w < wave; ++w) rank += wave_count[w * lists + mine];
+            const int at = histogram[mine] + rank;
+            a.token_indices[at] = d / a.slots;
+            a.draw_indices[at] = d;
+            if (a.weights_by_position != nullptr) a.weights_by_position[at] = a.weights_by_draw[d];
+        }
+        if (a.shared_tokens > 0) {
+            const int base = histogram[a.experts];
+            for (int t = threadIdx.x; t < a.shared_tokens; t += blockDim.x) {
+                a.token_indices[base + t] = t;
+                a.draw_indices[base + t] = a.draws + t;
+                if (a.weights_by_position != nullptr) a.weights_by_position[base + t] = 1.0f;
+            }
+        }
     }
 }
 
@@ -145,7 +195,12 @@ int launch_permutation(const PermutationArgs& args, hipStream_t stream) {
     if (a.slots > 1 && static_cast<uint64_t>(a.draws) * a.slots < (1ull << 32)) {
         a.slots_reciprocal = static_cast<unsigned>(((1ull << 32) + a.slots - 1) / a.slots);
     }
-    permutation_offsets_kernel<<<1, 1024, 0, stream>>>(a);
+    if (a.draws <= kFusedScatterDraws) {
+        permutation_offsets_kernel<true><<<1, 1024, 0, stream>>>(a);
+        AEON_LAUNCH_CHECK();
+        return AEON_OK;
+    }
+    permutation_offsets_kernel<false><<<1, 1024, 0, stream>>>(a);
     AEON_LAUNCH_CHECK();
     const int lists = a.experts + (a.shared_tokens > 0 ? 1 : 0);
     permutation_scatter_kernel<<<(lists + 3) / 4, 256, 0, stream>>>(a);
