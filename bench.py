@@ -303,8 +303,8 @@ def main():
                     help="also report batch 1/8/32/64 in the `sweep` field")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build measures one GPU's share of the path; run with --gpus 1 "
-                 "(how the path would shard is described in DESIGN.md)")
+        sys.exit("bench.py: this build measures one GPU's share of the path and uses no second GPU "
+                 "(no collectives, no sharding): run with --gpus 1")
 
     import numpy as np
     import torch

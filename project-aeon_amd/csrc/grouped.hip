@@ -9,8 +9,10 @@
 //     v_mfma_f32_16x16x32_f16 and multiplies by the row's fp16 scale (one rounding per weight,
 //     as the reference's grouped feed does); the fragment is then reused for every token tile
 //     of the window, which is what makes the dequantisation cheap next to the MFMAs;
-//   * token tiles past the tile's live count are skipped, so an expert with a handful of
-//     tokens costs its weight stream and little else.
+//   * the window's live count picks the body: 1, 2 or 4 token tiles with a deep ring of K
+//     groups in flight (grouped_run: bound by the latency of the weight stream), or the full
+//     window of 8 in a hand-pipelined body (grouped_run_full: bound by arithmetic), so an
+//     expert with a handful of tokens costs its weight stream and little else.
 // Weights are read once per (expert, position tile); tiles of one expert are adjacent in the
 // grid so their re-reads meet in L2 / Infinity Cache.
 #include <type_traits>

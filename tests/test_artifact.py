@@ -1,4 +1,4 @@
-"""The `.aeon` expert container reader (SURVEY "next" row: artifact reader + load-time repack).
+"""The `.aeon` expert container reader and the load-time repack into the resident pool.
 The container is written here with the writer's own format statement
 (scripts/convert_safetensors_to_aeon.py:463-486: "<12sIIIQ" header, "<QQ" entries); the reader's
 checks are the ones AeonModelLoader::open_experts makes (aeon_loader.hpp:345-405)."""
