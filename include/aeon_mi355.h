@@ -113,6 +113,18 @@ int aeon_moe_gemv_w13_swiglu(const void* d_activation, const aeon_w13_table* wei
 int aeon_moe_fused_w2_contrib(const void* d_expert_hidden, const aeon_w2_table* weights,
                               const float* d_topk_weights, float* d_contrib, int expert_count,
                               int N, int K, int rpw, int lpr, void* stream);
+
+/* The one-launch accumulation control, aeon_moe_fused_w2_accum_kernel + dispatch
+ * (aeon_moe_fused_w2.hpp:73-174): output_f32[row] += sum over e of topk_w[e] * (W2_e . hidden_e)[row]
+ * (+ initial_output[row] with e = 0 when given), output_f16[row] = half(output_f32[row]). The
+ * reference adds with atomicAdd in the scheduler's order and keeps per-block completion
+ * counters; here one workgroup owns a row block and walks the experts in slot order, so the
+ * result is reproducible and no counters are needed (the caller's stay untouched, i.e. at the
+ * zero the reference leaves them at). */
+int aeon_moe_fused_w2_accum(const void* d_expert_hidden, const aeon_w2_table* weights,
+                            const float* d_topk_weights, const void* d_initial_output,
+                            float* d_output_f32, void* d_output_f16, int expert_count, int N,
+                            int K, int rpw, int lpr, void* stream);
 /* moe_accumulate_fixed_order_kernel launch, src/platform/ops/moe_accumulate.hpp:73-92:
  * out[i] = half(float(shared[i]) + sum_{e ascending} contrib[e*hidden+i]); `d_shared` may be
  * NULL and may alias `d_out`. */

@@ -14,14 +14,15 @@ namespace aeon355 {
 constexpr int kWaves = 4;            // waves per workgroup = K splits
 constexpr int kMaxItersPerLane = 8;  // iterations one lane may own (K <= 8*kWaves*2*LPR*32)
 
-enum class SwzMode { Gemv, Dual, GateUp, W2Contrib };
+enum class SwzMode { Gemv, Dual, GateUp, W2Contrib, W2Accum };
 
 struct SwzArgs {
     const uint16_t* activation;  // fp16 bits
     aeon_w13_table w13;          // GateUp (w1/s1/w3/s3); Gemv/Dual use slot 0
     aeon_w2_table w2;            // W2Contrib
     const float* topk_weights;
-    uint16_t* out_a;  // Gemv/Dual output a, GateUp expert_hidden
+    const uint16_t* initial;  // W2Accum: optional fp16 row added with the first expert
+    uint16_t* out_a;  // Gemv/Dual output a, GateUp expert_hidden, W2Accum fp16 output
     uint16_t* out_b;  // Dual output b
     float* out_f32;   // W2Contrib contrib; GateUp optional zero-fill target
     int zero_dim;
@@ -46,7 +47,12 @@ __global__ __launch_bounds__(kWaves * 64) void swizzled_decode_kernel(SwzArgs a)
     static_assert(RPW * LPR == 32, "RPW and LPR describe one 32-slot storage tile");
     constexpr bool kTwo = (MODE == SwzMode::Dual || MODE == SwzMode::GateUp);
 
-    const int expert = blockIdx.y;
+    // W2Accum walks the experts itself, in slot order, so that the sum into the shared row has
+    // one writer and a fixed order; every other mode takes its expert from the grid.
+    constexpr bool kAccum = MODE == SwzMode::W2Accum;
+    constexpr bool kW2 = MODE == SwzMode::W2Contrib || kAccum;
+    const int first_expert = kAccum ? 0 : blockIdx.y;
+    const int last_expert = kAccum ? a.expert_count : first_expert + 1;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int half_id = lane >> 5;
@@ -54,7 +60,13 @@ __global__ __launch_bounds__(kWaves * 64) void swizzled_decode_kernel(SwzArgs a)
     const int row_block = blockIdx.x;
     const int row_in_block = lane32 / LPR;
     const int slice = lane32 % LPR;
+    __shared__ float partial[2][kWaves][RPW];
+    float running = 0.0f;  // W2Accum: the row's sum so far (threads below RPW)
+    if (kAccum && threadIdx.x < RPW && row_block * RPW + threadIdx.x < a.N) {
+        running = a.out_f32[row_block * RPW + threadIdx.x];
+    }
 
+    for (int expert = first_expert; expert < last_expert; ++expert) {
     if (MODE == SwzMode::GateUp && expert == 0 && a.out_f32 != nullptr) {
         for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < a.zero_dim;
              i += gridDim.x * blockDim.x) {
@@ -67,7 +79,7 @@ __global__ __launch_bounds__(kWaves * 64) void swizzled_decode_kernel(SwzArgs a)
     const uint4* pb = nullptr;
     const uint16_t* sb = nullptr;
     const uint16_t* x = a.activation;
-    if (MODE == SwzMode::W2Contrib) {
+    if (kW2) {
         pa = static_cast<const uint4*>(a.w2.w2[expert]);
         sa = static_cast<const uint16_t*>(a.w2.s2[expert]);
         x += static_cast<size_t>(expert) * (static_cast<size_t>(a.iterations) * LPR * 32);
@@ -115,7 +127,6 @@ __global__ __launch_bounds__(kWaves * 64) void swizzled_decode_kernel(SwzArgs a)
     acc_a = wave_xor_sum(acc_a, (LPR - 1) | 32);
     if (kTwo) acc_b = wave_xor_sum(acc_b, (LPR - 1) | 32);
 
-    __shared__ float partial[2][kWaves][RPW];
     if (half_id == 0 && slice == 0) {
         partial[0][wave][row_in_block] = acc_a;
         if (kTwo) partial[1][wave][row_in_block] = acc_b;
@@ -139,10 +150,20 @@ __global__ __launch_bounds__(kWaves * 64) void swizzled_decode_kernel(SwzArgs a)
             } else if (MODE == SwzMode::GateUp) {
                 a.out_a[static_cast<size_t>(expert) * a.N + row] =
                     float_to_half_bits(clamped_swiglu(sum_a, sum_b, a.limit));
-            } else {
+            } else if (MODE == SwzMode::W2Contrib) {
                 a.out_f32[static_cast<size_t>(expert) * a.N + row] = a.topk_weights[expert] * sum_a;
+            } else {
+                float contribution = a.topk_weights[expert] * sum_a;
+                if (expert == 0 && a.initial != nullptr) contribution += half_bits_to_float(a.initial[row]);
+                running += contribution;
+                if (expert == last_expert - 1) {
+                    a.out_f32[row] = running;
+                    a.out_a[row] = float_to_half_bits(running);
+                }
             }
         }
+    }
+    if (kAccum) __syncthreads();  // the exchange buffer is reused by the next expert
     }
 }
 
@@ -296,6 +317,34 @@ extern "C" int aeon_moe_fused_w2_contrib(const void* d_expert_hidden, const aeon
     a.N = N;
     a.iterations = K / (lpr * 32);
     return launch<SwzMode::W2Contrib>(a, rpw, lpr, expert_count, as_stream(stream), who);
+}
+
+extern "C" int aeon_moe_fused_w2_accum(const void* d_expert_hidden, const aeon_w2_table* weights,
+                                       const float* d_topk_weights, const void* d_initial_output,
+                                       float* d_output_f32, void* d_output_f16, int expert_count,
+                                       int N, int K, int rpw, int lpr, void* stream) {
+    const char* who = "aeon_moe_fused_w2_accum";
+    AEON_REQUIRE(d_expert_hidden && weights && d_topk_weights && d_output_f32 && d_output_f16,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
+    AEON_REQUIRE(expert_count > 0 && expert_count <= AEON_SWIZZLED_MAX_EXPERTS,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: expert_count %d outside 1..%d", who, expert_count,
+                 AEON_SWIZZLED_MAX_EXPERTS);
+    if (int rc = check_shape(N, K, rpw, lpr, who)) return rc;
+    for (int e = 0; e < expert_count; ++e) {
+        AEON_REQUIRE(weights->w2[e] && weights->s2[e], AEON_ERR_INVALID_ARGUMENT,
+                     "%s: expert slot %d has a null weight pointer", who, e);
+    }
+    SwzArgs a{};
+    a.activation = static_cast<const uint16_t*>(d_expert_hidden);
+    a.w2 = *weights;
+    a.topk_weights = d_topk_weights;
+    a.initial = static_cast<const uint16_t*>(d_initial_output);
+    a.out_f32 = d_output_f32;
+    a.out_a = static_cast<uint16_t*>(d_output_f16);
+    a.expert_count = expert_count;
+    a.N = N;
+    a.iterations = K / (lpr * 32);
+    return launch<SwzMode::W2Accum>(a, rpw, lpr, 1, as_stream(stream), who);
 }
 
 extern "C" int aeon_moe_accumulate_fixed_order(const float* d_contrib, int expert_count,

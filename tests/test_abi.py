@@ -57,6 +57,13 @@ def test_argument_errors_without_device_work():
         capi.call("aeon_a64_gemv", one, 256, one, one, one, 40, 1, 40, 256, None)
     with pytest.raises(ValueError, match="tokens"):
         capi.call("aeon_a64_gemv", one, 256, one, one, one, 64, 9, 64, 256, None)
+    w2 = capi.W2Table()
+    with pytest.raises(ValueError, match="expert_count"):
+        capi.call("aeon_moe_fused_w2_accum", one, C.byref(w2), one, None, one, one, 0, 4096, 2048,
+                  8, 4, None)
+    with pytest.raises(ValueError, match="null weight pointer"):
+        capi.call("aeon_moe_fused_w2_accum", one, C.byref(w2), one, None, one, one, 2, 4096, 2048,
+                  8, 4, None)
     with pytest.raises(ValueError, match="the sink holds"):
         capi.call("aeon_calibrate_mfma_f16", 1, 10, 4, one, C.c_size_t(512), None, None)
     assert capi.lib().aeon_last_error() != b""

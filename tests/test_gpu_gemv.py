@@ -204,6 +204,28 @@ def test_swizzled_expert_trio_reference_shapes(orc, experts):
     assert torch.equal(out, acc.half())
     want_out = orc.moe_combine(want_contrib, shared.cpu().numpy().astype(np.float64))
     assert h.rel_err(out.cpu().numpy(), want_out) <= TOL
+    # the one-launch accumulation control (aeon_moe_fused_w2.hpp:73-174): the same slot-order
+    # sum from a zeroed row, so bit-identical to contrib + reduce without an initial row, and
+    # within tolerance of the oracle with the shared row entering beside the first expert
+    acc32 = torch.zeros(H, dtype=torch.float32, device="cuda")
+    acc16 = torch.zeros(H, dtype=torch.float16, device="cuda")
+    capi.call("aeon_moe_fused_w2_accum", capi.vp(hidden), C.byref(w2), capi.vp(d_w), None,
+              capi.vp(acc32), capi.vp(acc16), experts, H, I, 8, 4, h.stream_ptr())
+    plain = torch.zeros(H, dtype=torch.float32, device="cuda")
+    for e in range(experts):
+        plain = plain + contrib[e]
+    assert torch.equal(acc32, plain) and torch.equal(acc16, plain.half())
+    acc32.zero_()
+    capi.call("aeon_moe_fused_w2_accum", capi.vp(hidden), C.byref(w2), capi.vp(d_w),
+              capi.vp(shared), capi.vp(acc32), capi.vp(acc16), experts, H, I, 8, 4,
+              h.stream_ptr())
+    assert h.rel_err(acc16.cpu().numpy(), want_out) <= TOL
+    # it adds to what the row holds: a second call doubles the routed part
+    capi.call("aeon_moe_fused_w2_accum", capi.vp(hidden), C.byref(w2), capi.vp(d_w), None,
+              capi.vp(acc32), capi.vp(acc16), experts, H, I, 8, 4, h.stream_ptr())
+    twice = orc.moe_combine(np.concatenate([want_contrib, want_contrib]),
+                            shared.cpu().numpy().astype(np.float64))
+    assert h.rel_err(acc32.cpu().numpy(), twice) <= TOL
 
 
 @pytest.mark.parametrize("use_mfma", [0, 1])
