@@ -84,3 +84,63 @@ def test_shim_headers_and_cpp_gates_compile():
         subprocess.run(["/opt/rocm/bin/hipcc", "--offload-arch=gfx950", "-std=c++20", "-x", "hip",
                         "-fsyntax-only", "-I", shim, "-I", os.path.join(ROOT, "include"), src],
                        check=True, stderr=subprocess.DEVNULL)
+
+
+def test_shim_cpu_router_matches_the_oracle(tmp_path):
+    """cpu_moe_router of the router shim header (host code) against the fp64 oracle, itself
+    pinned to the reference's host oracle: the fixture of tests/test_moe_router.cpp:28-35
+    (logit ((i % 31) - 15) * 0.2, bias ((i % 17) - 8) * 0.05, many exact ties) and seeded
+    random logits; ids equal position by position, weights to 1e-6."""
+    import subprocess
+    import sys
+    import numpy as np
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import orc
+    src = tmp_path / "r.cpp"
+    src.write_text('''
+#include "architecture/deepseek_v4/kernels/moe_router.hpp"
+#include <cstdio>
+int main(int argc, char** argv) {
+    int tokens = 0, experts = 0, top_k = 0; float scaling = 0;
+    std::FILE* f = std::fopen(argv[1], "rb");
+    if (!f || std::fread(&tokens, 4, 1, f) != 1 || std::fread(&experts, 4, 1, f) != 1 ||
+        std::fread(&top_k, 4, 1, f) != 1 || std::fread(&scaling, 4, 1, f) != 1) return 2;
+    std::vector<float> logits(size_t(tokens) * experts), bias(experts);
+    if (std::fread(logits.data(), 4, logits.size(), f) != logits.size()) return 3;
+    if (std::fread(bias.data(), 4, bias.size(), f) != bias.size()) return 4;
+    std::vector<float> w(size_t(tokens) * top_k);
+    std::vector<int32_t> ids(size_t(tokens) * top_k);
+    aeon::kernel::cpu_moe_router(logits.data(), bias.data(), nullptr, nullptr, w.data(), ids.data(),
+                                 tokens, experts, top_k, scaling, true);
+    for (size_t i = 0; i < ids.size(); ++i) std::printf("%d %.9g\\n", ids[i], w[i]);
+    return 0;
+}
+''')
+    exe = tmp_path / "r"
+    subprocess.run(["/opt/rocm/bin/hipcc", "--offload-arch=gfx950", "-std=c++20",
+                    "-x", "hip", "-O1", "-I", os.path.join(ROOT, "project-aeon_amd", "shim"),
+                    str(src), "-o", str(exe)], check=True, stderr=subprocess.DEVNULL)
+    rng = np.random.default_rng(5)
+    cases = []
+    i = np.arange(4 * 256)
+    cases.append((((i % 31) - 15) * np.float32(0.2), ((np.arange(256) % 17) - 8) * np.float32(0.05),
+                  4, 256, 6, 1.5))
+    cases.append((rng.normal(0, 2, 8 * 256).astype(np.float32),
+                  rng.normal(0, 0.1, 256).astype(np.float32), 8, 256, 8, 1.0))
+    for logits, bias, tokens, experts, top_k, scaling in cases:
+        logits = logits.astype(np.float32).reshape(tokens, experts)
+        bias = bias.astype(np.float32)
+        blob = tmp_path / "in.bin"
+        with open(blob, "wb") as f:
+            f.write(np.array([tokens, experts, top_k], dtype=np.int32).tobytes())
+            f.write(np.array([scaling], dtype=np.float32).tobytes())
+            f.write(logits.tobytes())
+            f.write(bias.tobytes())
+        out = subprocess.run([str(exe), str(blob)], capture_output=True, text=True, check=True).stdout
+        rows = [line.split() for line in out.strip().splitlines()]
+        got_ids = np.array([int(r[0]) for r in rows]).reshape(tokens, top_k)
+        got_w = np.array([float(r[1]) for r in rows]).reshape(tokens, top_k)
+        for t in range(tokens):
+            ids, w = orc.router_topk(logits[t], bias, top_k, scaling, 0)
+            assert np.array_equal(got_ids[t], ids)
+            assert np.max(np.abs(got_w[t] - w)) <= 1e-6
