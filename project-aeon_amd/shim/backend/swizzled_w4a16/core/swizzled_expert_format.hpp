@@ -4,6 +4,8 @@
 // are the reference's for hidden 4096 / intermediate 2048
 // (src/backend/swizzled_w4a16/core/swizzled_expert_format.hpp:9-30); swizzled_expert_layout()
 // states the same order for any shape.
+#include "infrastructure/expert/storage/expert_format.hpp"
+
 #include <cstddef>
 #include <cstdint>
 
@@ -40,5 +42,6 @@ static_assert(AEON_W1_SCALE_OFFSET == 4194304 && AEON_W2_PACKED_OFFSET == 471859
               AEON_W2_SCALE_OFFSET == 8912896 && AEON_W3_PACKED_OFFSET == 9437184 &&
               AEON_W3_SCALE_OFFSET == 13631488 && AEON_SWIZZLED_EXPERT_BYTES == 14155776,
               "the reference's published offsets");
+static_assert(AEON_SWIZZLED_EXPERT_BYTES == AEON_EXPERT_BYTES, "one payload size, two names");
 
 }  // namespace aeon::core

@@ -3,7 +3,9 @@ against this repository's shim headers and linked to libaeon_mi355.so (oracle/Ma
 `gates`; the binaries live in oracle/_ref/gates and travel prebuilt): tests/test_w4a16_swizzle.cpp
 on the CPU, tests/test_w4a16_swizzled_gemv.cpp, test_w4a16_swizzled_dual_gemv.cpp,
 test_moe_grouped_batch_parity.cpp, test_expert_permutation.cpp, test_aeon_moe_fused_w2.cpp,
-test_moe_router.cpp and test_hc_sinkhorn.cpp on the GPU. They are the
+test_moe_router.cpp, test_hc_sinkhorn.cpp, test_v4_hc_oracle.cpp and
+test_v4_grouped_wmma_oracle.cpp on the GPU (the last two hold the kernels to the reference's own
+host oracle, reference/dsv4_oracle.hpp, compiled in from the reference tree). They are the
 drop-in check: the entry points keep the reference's names, signatures and error behaviour, and
 the reference's own assertions hold on the gfx950 kernels behind them."""
 import os
@@ -35,6 +37,7 @@ def test_reference_swizzle_gate_on_cpu():
 @pytest.mark.gpu
 @pytest.mark.parametrize("gate", ["test_w4a16_swizzled_gemv", "test_w4a16_swizzled_dual_gemv",
                                   "test_moe_grouped_batch_parity", "test_expert_permutation",
-                                  "test_aeon_moe_fused_w2", "test_moe_router", "test_hc_sinkhorn"])
+                                  "test_aeon_moe_fused_w2", "test_moe_router", "test_hc_sinkhorn",
+                                  "test_v4_hc_oracle", "test_v4_grouped_wmma_oracle"])
 def test_reference_gate_on_gpu(gate):
     _run(gate)
