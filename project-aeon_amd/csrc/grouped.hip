@@ -9,10 +9,11 @@
 //     v_mfma_f32_16x16x32_f16 and multiplies by the row's fp16 scale (one rounding per weight,
 //     as the reference's grouped feed does); the fragment is then reused for every token tile
 //     of the window, which is what makes the dequantisation cheap next to the MFMAs;
-//   * the window's live count picks the body: 1, 2 or 4 token tiles with a deep ring of K
-//     groups in flight (grouped_run: bound by the latency of the weight stream), or the full
-//     window of 8 in a hand-pipelined body (grouped_run_full: bound by arithmetic), so an
-//     expert with a handful of tokens costs its weight stream and little else.
+//   * the window's live count picks the body: 1, 2, 3 or 4 token tiles with a deep ring of K
+//     groups in flight (grouped_run: bound by the latency of the weight stream), or 6 or 8 in
+//     a hand-pipelined body (grouped_run_full: bound by arithmetic), so an expert with a
+//     handful of tokens costs its weight stream and little else and no window computes more
+//     than two token tiles of padding.
 // Weights are read once per (expert, position tile); tiles of one expert are adjacent in the
 // grid so their re-reads meet in L2 / Infinity Cache.
 #include <type_traits>
@@ -241,8 +242,8 @@ __device__ __forceinline__ void grouped_run(const SegGateUpArgs& gu, const SegDo
     }
 }
 
-// The body for a full window (eight token tiles), where arithmetic bounds the time. A K group is
-// 32 blocks; block (st, mt) is the NM*R MFMAs of MFMA step st on token tile mt. VALU work hides
+// The body for a wide window (six or eight token tiles), where arithmetic bounds the time. A K
+// group is 4*LIVE blocks; block (st, mt) is the NM*R MFMAs of MFMA step st on token tile mt. VALU work hides
 // behind the matrix pipe only when the same wave issues it right after an MFMA, so the group is
 // software-pipelined by hand, block by block:
 //   * the B fragments of a pair of blocks are read from LDS one pair early;
@@ -250,11 +251,11 @@ __device__ __forceinline__ void grouped_run(const SegGateUpArgs& gu, const SegDo
 //     unpacked one fragment per two blocks, behind the MFMAs of step st;
 //   * a scheduling fence after every block keeps the compiler from regrouping any of it.
 // One K group of weights and activations is in flight while one is computed (two ring slots).
-template <bool GATE_UP, int R>
+template <bool GATE_UP, int R, int LIVE>
 __device__ __forceinline__ void grouped_run_full(const SegGateUpArgs& gu, const SegDownArgs& dn,
                                                  const aeon_a64_expert& e, int first, int count,
                                                  half8_t* xs_flat) {
-    constexpr int LIVE = kGroupedMT;
+    static_assert(LIVE % 2 == 0 && LIVE <= kGroupedMT, "blocks go in pairs");
     constexpr int NM = GATE_UP ? 2 : 1;
     constexpr int kFrags = NM * R;
     constexpr int kBufferStride = LIVE * 4 * 64;  // in 16-byte units
@@ -395,10 +396,15 @@ __device__ __forceinline__ void grouped_run_full(const SegGateUpArgs& gu, const 
                 for (int r = 0; r < R; ++r)
                     acc[m][r][mt + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[st % 2][m][r], b[(i + 1) % 4],
                                                                                 acc[m][r][mt + 1], 0, 0, 0);
-            {
-                const int f = mt / 2, m = f / R, r = f % R;
-                a[(st + 1) % 2][m][r] = st < 3 ? scaled_fragment(wq[s][m][r][st < 3 ? st + 1 : 0], scale_pair(sc[s][m][r]))
-                                      : scaled_fragment(wq[sn][m][r][0], scale_pair(sc[sn][m][r]));
+            // this pair's share of the four fragments of the next MFMA step
+#pragma unroll
+            for (int f = 0; f < kFrags; ++f) {
+                if (f * (LIVE / 2) / kFrags == mt / 2) {
+                    const int m = f / R, r = f % R;
+                    a[(st + 1) % 2][m][r] =
+                        st < 3 ? scaled_fragment(wq[s][m][r][st < 3 ? st + 1 : 0], scale_pair(sc[s][m][r]))
+                               : scaled_fragment(wq[sn][m][r][0], scale_pair(sc[sn][m][r]));
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -464,10 +470,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     __shared__ half8_t xs[2 * kGroupedMT * 4 * 64];
 
     const int live_tiles = (count + 15) >> 4;
-    if (live_tiles > 4) {
-        grouped_run_full<GATE_UP, R>(gu, dn, e, first, count, xs);
-    } else if (live_tiles > 2) {
+    if (live_tiles > 6) {
+        grouped_run_full<GATE_UP, R, 8>(gu, dn, e, first, count, xs);
+    } else if (live_tiles > 4) {
+        grouped_run_full<GATE_UP, R, 6>(gu, dn, e, first, count, xs);
+    } else if (live_tiles > 3) {
         grouped_run<GATE_UP, R, 4, 3>(gu, dn, e, first, count, xs);
+    } else if (live_tiles > 2) {
+        grouped_run<GATE_UP, R, 3, 3>(gu, dn, e, first, count, xs);
     } else if (live_tiles > 1) {
         grouped_run<GATE_UP, R, 2, 3>(gu, dn, e, first, count, xs);
     } else {

@@ -298,6 +298,38 @@ def test_prefill_grouped_small_full_oracle(orc):
     assert np.array_equal(again, out)
 
 
+def test_prefill_window_bodies_at_every_live_count(orc):
+    """One expert per window size class and its edges: the grouped kernel picks a body by the
+    window's live token tiles (1, 2, 3, 4, 6 or 8 of 16 positions), so experts are given exactly
+    1, 15, 16, 17, ... 128, 129 and 200 tokens (top-1 routing makes the counts exact) and every
+    token is checked against the oracle."""
+    torch, h, capi, moe, synth = _setup()
+    H, I, limit = 512, 256, 7.0
+    counts = [1, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64, 65, 80, 95, 96, 97, 111, 112, 113, 127,
+              128, 129, 200]
+    E, T = len(counts), sum(counts)
+    pool = moe.ExpertPool(E, H, I)
+    assert pool.fill_synthetic(seed=21, first_expert_id=0) == 0
+    layer = moe.MoeLayer(pool, E, 1, False, limit)
+    rng = np.random.default_rng(21)
+    ids = np.repeat(np.arange(E, dtype=np.int32), counts)
+    rng.shuffle(ids)
+    ids = ids.reshape(T, 1)
+    w = (0.25 + rng.random((T, 1))).astype(np.float32)
+    x = synth.activations(21, T, H)
+    out = layer.routed(h.dev_half(x), h.to_dev(ids), h.to_dev(w))
+    torch.cuda.synchronize()
+    out = out.cpu().numpy()
+    experts = {e: h.Expert(21, e, H, I) for e in range(E)}
+    want = _oracle_layer(orc, h, experts, x, ids, w, None, limit)
+    peak = np.abs(want).max()
+    assert peak > 0.1
+    for e in range(E):
+        rows = np.nonzero(ids[:, 0] == e)[0]
+        assert len(rows) == counts[e]
+        assert np.abs(out[rows] - want[rows]).max() <= 6e-3 * peak, (e, counts[e])
+
+
 def test_config3_prefill_full_size_sampled(orc):
     """BASELINE config 3 at full size: 2048 tokens, top-8 of 256 experts with Zipf(1.1)
     popularity, H=7168, I=2048, + shared expert. The oracle covers a sample of tokens; the rest
