@@ -139,7 +139,9 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
                            (draws < layer->experts ? draws : layer->experts);
     // Many live segments: the wide kernels (k_split 0: four waves per workgroup sharing the
     // activations through LDS, no K split). Few: split K four ways so the chip still fills.
-    const int split_gate = live_bound * (layer->intermediate / 16) >= 8192 ? 0 : 4;
+    // Measured at H 7168 / I 2048: the gate/up launch is faster K-split up to batch 2 (17 live
+    // lists) and wide from batch 4 (33) on; the down launch is faster wide at every batch.
+    const int split_gate = live_bound * (layer->intermediate / 16) >= 3072 ? 0 : 4;
     const int split_down = live_bound * (layer->hidden / 16) >= 4000 ? 0 : 4;
     // Wide form: 64 gate/up rows or 128 down rows per workgroup and four (three) K groups of
     // weights in flight per wave measured best at batch 64 on both a concentrated and a spread

@@ -131,11 +131,13 @@ class MoeLayer:
         return self.workspace
 
     def decode(self, x, out=None, ids=None, weights=None):
-        """x fp16 [tokens][hidden] -> (out fp16 [tokens][hidden], ids int32, weights fp32)."""
+        """x fp16 [tokens][hidden] -> (out fp16 [tokens][hidden], ids int32, weights fp32).
+        Without an always-on expert the routed sum is added to what `out` holds, so an `out`
+        allocated here starts at zero."""
         tokens = x.shape[0]
         ws = self._workspace(tokens)
         k = self.cfg.top_k
-        out = torch.empty_like(x) if out is None else out
+        out = torch.zeros_like(x) if out is None else out
         ids = torch.empty(tokens, k, dtype=torch.int32, device=x.device) if ids is None else ids
         weights = (torch.empty(tokens, k, dtype=torch.float32, device=x.device)
                    if weights is None else weights)
@@ -145,10 +147,12 @@ class MoeLayer:
         return out, ids, weights
 
     def routed(self, x, ids, weights, out=None):
-        """The expert part only, for given routing (ids int32 / weights fp32 [tokens][top_k])."""
+        """The expert part only, for given routing (ids int32 / weights fp32 [tokens][top_k]).
+        A layer without an always-on expert adds the routed sum to what `out` holds (the
+        reference's in-place accumulator); an `out` allocated here therefore starts at zero."""
         tokens = x.shape[0]
         ws = self._workspace(tokens)
-        out = torch.empty_like(x) if out is None else out
+        out = torch.zeros_like(x) if out is None else out
         capi.call("aeon_moe_layer_routed", C.byref(self.cfg), capi.vp(x), x.stride(0), tokens,
                   capi.vp(ids), capi.vp(weights), capi.vp(out), out.stride(0), capi.vp(ws),
                   C.c_size_t(ws.numel()), stream_ptr())
