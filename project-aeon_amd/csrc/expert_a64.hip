@@ -621,31 +621,49 @@ int launch_seg_down(const SegDownArgs& a, int k_split, int row_tiles, int depth,
 // Fixed-order reduce over a token's slots
 // ---------------------------------------------------------------------------------------------
 
+// Four columns per thread (hidden is a multiple of 128): 16-byte loads of the fp32 contributions.
 __global__ __launch_bounds__(256) void token_reduce_kernel(
     const float* __restrict__ contrib, int slots, int shared_base, const uint16_t* initial,
     long initial_stride, uint16_t* out, long out_stride, int hidden) {
     const int t = blockIdx.y;
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    const int i = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (i >= hidden) return;
-    float acc = 0.0f;
+    float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
     if (shared_base >= 0) {
         // The shared expert enters as an fp16 value, as it does when a separate pass has
         // stored it into the token's accumulator first.
-        acc = half_bits_to_float(float_to_half_bits(
-            contrib[static_cast<size_t>(shared_base + t) * hidden + i]));
+        const float4_t v = *reinterpret_cast<const float4_t*>(
+            contrib + static_cast<size_t>(shared_base + t) * hidden + i);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[q] = half_bits_to_float(float_to_half_bits(v[q]));
     } else if (initial != nullptr) {
-        acc = half_bits_to_float(initial[t * initial_stride + i]);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[q] = half_bits_to_float(initial[t * initial_stride + i + q]);
     }
     const float* c = contrib + static_cast<size_t>(t) * slots * hidden + i;
-    for (int s = 0; s < slots; ++s) acc += c[static_cast<size_t>(s) * hidden];
-    out[t * out_stride + i] = float_to_half_bits(acc);
+    for (int s = 0; s < slots; ++s) {
+        const float4_t v = *reinterpret_cast<const float4_t*>(c + static_cast<size_t>(s) * hidden);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[q] += v[q];
+    }
+    uint16_t* o = out + t * out_stride + i;
+    if ((reinterpret_cast<uintptr_t>(o) & 7) == 0) {
+        uint2 packed;
+        packed.x = float_to_half_bits(acc[0]) | (static_cast<uint32_t>(float_to_half_bits(acc[1])) << 16);
+        packed.y = float_to_half_bits(acc[2]) | (static_cast<uint32_t>(float_to_half_bits(acc[3])) << 16);
+        *reinterpret_cast<uint2*>(o) = packed;
+    } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) o[q] = float_to_half_bits(acc[q]);
+    }
 }
 
 int launch_token_reduce(const float* contrib, int tokens, int slots, int shared_base,
                         const uint16_t* initial, long initial_stride, uint16_t* out,
                         long out_stride, int hidden, hipStream_t stream) {
     if (tokens <= 0) return AEON_OK;
-    token_reduce_kernel<<<dim3((hidden + 255) / 256, tokens), 256, 0, stream>>>(
+    AEON_REQUIRE(hidden % 4 == 0, AEON_ERR_INVALID_ARGUMENT, "token reduce: hidden %d is not a multiple of 4", hidden);
+    token_reduce_kernel<<<dim3((hidden / 4 + 255) / 256, tokens), 256, 0, stream>>>(
         contrib, slots, shared_base, initial, initial_stride, out, out_stride, hidden);
     AEON_LAUNCH_CHECK();
     return AEON_OK;
