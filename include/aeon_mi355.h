@@ -130,6 +130,12 @@ int aeon_moe_fused_w2_accum(const void* d_expert_hidden, const aeon_w2_table* we
  * NULL and may alias `d_out`. */
 int aeon_moe_accumulate_fixed_order(const float* d_contrib, int expert_count,
                                     const void* d_shared, void* d_out, int hidden, void* stream);
+/* The same reduce for every token of a chunk in one launch, in place of the per-token launches
+ * of run_moe_grouped_expert_batch (src/architecture/deepseek_v4/moe/moe_grouped_batch.hpp:136-146):
+ * out[t][i] = half(float(out[t][i]) + sum_{s ascending} contrib[(t*slots + s)*hidden + i]), i.e.
+ * each token's row (pitch out_stride elements) is its own fp16 starting value. hidden % 4 == 0. */
+int aeon_moe_accumulate_fixed_order_tokens(const float* d_contrib, int tokens, int slots,
+                                           void* d_out, int out_stride, int hidden, void* stream);
 /* v4_swiglu_clamp_kernel launch, src/architecture/deepseek_v4/kernels/v4_swiglu_clamp.hpp:18-34. */
 int aeon_swiglu_clamp(const void* d_gate, const void* d_up, void* d_out, int total_elements,
                       float limit, void* stream);

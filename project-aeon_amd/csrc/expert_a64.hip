@@ -673,6 +673,19 @@ int launch_token_reduce(const float* contrib, int tokens, int slots, int shared_
 
 using namespace aeon355;
 
+extern "C" int aeon_moe_accumulate_fixed_order_tokens(const float* d_contrib, int tokens, int slots,
+                                                      void* d_out, int out_stride, int hidden,
+                                                      void* stream) {
+    const char* who = "aeon_moe_accumulate_fixed_order_tokens";
+    AEON_REQUIRE(d_contrib && d_out, AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
+    AEON_REQUIRE(tokens >= 0 && slots > 0 && hidden > 0 && hidden % 4 == 0 && out_stride >= hidden,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: bad shape (tokens=%d slots=%d hidden=%d pitch=%d)",
+                 who, tokens, slots, hidden, out_stride);
+    return launch_token_reduce(d_contrib, tokens, slots, -1, static_cast<const uint16_t*>(d_out),
+                               out_stride, static_cast<uint16_t*>(d_out), out_stride, hidden,
+                               as_stream(stream));
+}
+
 extern "C" int aeon_a64_gemv(const void* d_x, int x_stride, const void* d_packed,
                              const void* d_scale, void* d_out, int out_stride, int tokens, int N,
                              int K, void* stream) {

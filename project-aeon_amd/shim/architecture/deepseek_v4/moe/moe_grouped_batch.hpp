@@ -1,18 +1,24 @@
 #pragma once
-// run_moe_grouped_expert_batch and MoeGroupedBatchScratch with the reference's signatures
-// (src/architecture/deepseek_v4/moe/moe_grouped_batch.hpp:34-147): permutation, grouped gate/up
-// and W2 per range of at most kAeonSwizzledMaxExperts experts, then the per-token slot-ordered
-// reduce folding in whatever the caller already stored in each token's output row.
+// run_moe_grouped_expert_batch and MoeGroupedBatchScratch under the reference's names and
+// signatures (src/architecture/deepseek_v4/moe/moe_grouped_batch.hpp:34-147): a chunk's routing
+// goes through the token -> expert permutation, the grouped gate/up and W2 launches and the
+// slot-ordered reduce that folds in what the caller already stored in each token's output row.
 //
-// The Filler contract hands the host each expert's draw count, so the expert offsets are read
-// back and the stream synchronised once per call, as the reference does (:80-83); the
-// resident-expert path (aeon_moe_layer_routed) has no such read-back.
+// What the contract fixes: the Filler is told every expert's draw count, so the per-expert bounds
+// are read back once per call (one stream synchronisation, as at :80-83), a weight table holds
+// kAeonSwizzledMaxExperts experts, and an expert wider than the scratch is refused (:90-93).
+// What is done differently here:
+//   * the grouped launches read the permutation's own device-side bounds (the table of a launch
+//     is a window of perm_offsets, positions stay absolute), so nothing is re-based on the host
+//     and no bounds are copied back to the device; `batch_offsets` of the scratch is unused;
+//   * a window with no draws costs no launch and no Filler call;
+//   * the reduce is one launch over all tokens of the chunk, not one per token.
+// The resident-expert path (aeon_moe_layer_routed) needs none of this: it has no read-back.
 #include "architecture/deepseek_v4/kernels/moe_grouped_dispatch.hpp"
 #include "infrastructure/hip_check.hpp"
 #include "platform/ops/expert_permutation.hpp"
 #include "platform/ops/moe_accumulate.hpp"
 
-#include <algorithm>
 #include <cstddef>
 #include <cstdint>
 #include <stdexcept>
@@ -25,16 +31,16 @@ struct MoeGroupedBatchScratch {
     int* perm_tokens{nullptr};      // [token_count * slots]
     int* perm_draws{nullptr};       // [token_count * slots]
     float* perm_weights{nullptr};   // [token_count * slots]
-    int* batch_offsets{nullptr};    // [kAeonSwizzledMaxExperts + 1]
+    int* batch_offsets{nullptr};    // [kAeonSwizzledMaxExperts + 1], kept for the signature
     half* chunk_hidden{nullptr};    // [kAeonSwizzledMaxExperts, hidden_tokens, intermediate]
     float* chunk_contrib{nullptr};  // [token_count * slots, hidden]
     int intermediate{0};
     int hidden{0};
-    int hidden_tokens{0};  // rows of chunk_hidden per expert; a wider expert is refused
+    int hidden_tokens{0};  // rows of chunk_hidden per expert
 };
 
-// fill(expert, j, count, w13, w2) sets table position j for expert `expert`, which owns `count`
-// draws (0 = never read).
+// fill(expert, j, count, w13, w2) puts expert `expert`, which owns `count` draws, at position j
+// of the two weight tables; an expert with count 0 may leave its position empty.
 template <class Filler>
 void run_moe_grouped_expert_batch(const half* batch_input, int input_stride, const int* batch_ids,
                                   const float* batch_weights, uint32_t token_count, int slots,
@@ -42,57 +48,45 @@ void run_moe_grouped_expert_batch(const half* batch_input, int input_stride, con
                                   const MoeGroupedBatchScratch& scratch, Filler&& fill,
                                   half* batch_output, int output_stride, hipStream_t stream = 0) {
     if (token_count == 0) return;
-    kernel::dispatch_expert_permutation(batch_ids, static_cast<int>(token_count), slots,
-                                        expert_count, scratch.perm_offsets, scratch.perm_tokens,
+    const int tokens = static_cast<int>(token_count);
+    kernel::dispatch_expert_permutation(batch_ids, tokens, slots, expert_count,
+                                        scratch.perm_offsets, scratch.perm_tokens,
                                         scratch.perm_draws, batch_weights, scratch.perm_weights,
                                         stream);
-    std::vector<int> offsets(static_cast<size_t>(expert_count) + 1);
-    CHECK_HIP(hipMemcpyAsync(offsets.data(), scratch.perm_offsets, offsets.size() * sizeof(int),
+
+    std::vector<int> bound(static_cast<size_t>(expert_count) + 1);
+    CHECK_HIP(hipMemcpyAsync(bound.data(), scratch.perm_offsets, bound.size() * sizeof(int),
                              hipMemcpyDeviceToHost, stream));
     CHECK_HIP(hipStreamSynchronize(stream));
+    auto draws_of = [&](int expert) { return bound[expert + 1] - bound[expert]; };
 
     int widest = 1;
-    for (int e = 0; e < expert_count; ++e) widest = std::max(widest, offsets[e + 1] - offsets[e]);
+    for (int expert = 0; expert < expert_count; ++expert) {
+        if (draws_of(expert) > widest) widest = draws_of(expert);
+    }
     if (widest > scratch.hidden_tokens) {
         throw std::invalid_argument(
             "run_moe_grouped_expert_batch: the chunk's widest expert exceeds the scratch");
     }
 
-    const int per_launch = kernel::kAeonSwizzledMaxExperts;
-    for (int base = 0; base < expert_count; base += per_launch) {
-        const int batch_count = std::min(per_launch, expert_count - base);
-        if (offsets[base] == offsets[base + batch_count]) continue;  // no draws in this range
-        const int first_draw = offsets[base];
-        kernel::SwizzledW13ExpertPtrs w13{};
-        kernel::SwizzledW2ExpertPtrs w2{};
-        std::vector<int> rebased(static_cast<size_t>(batch_count) + 1);
-        for (int j = 0; j < batch_count; ++j) {
-            const int expert = base + j;
-            rebased[j] = offsets[expert] - first_draw;
-            fill(expert, j, offsets[expert + 1] - offsets[expert], w13, w2);
-        }
-        rebased[batch_count] = offsets[base + batch_count] - first_draw;
-        // pageable host memory: the copy is complete, as far as the host buffer goes, on return
-        CHECK_HIP(hipMemcpyAsync(scratch.batch_offsets, rebased.data(), rebased.size() * sizeof(int),
-                                 hipMemcpyHostToDevice, stream));
+    constexpr int kTable = kernel::kAeonSwizzledMaxExperts;
+    for (int window = 0; window < expert_count; window += kTable) {
+        const int in_window = expert_count - window < kTable ? expert_count - window : kTable;
+        if (bound[window + in_window] == bound[window]) continue;
+        kernel::SwizzledW13ExpertPtrs gate_up{};
+        kernel::SwizzledW2ExpertPtrs down{};
+        for (int j = 0; j < in_window; ++j) fill(window + j, j, draws_of(window + j), gate_up, down);
+        const int* device_bounds = scratch.perm_offsets + window;  // absolute positions
         kernel::dispatch_aeon_moe_grouped_w13_swiglu_wmma<4, 4, 8, kernel::kMoeGroupedMTiles>(
-            batch_input, scratch.batch_offsets, scratch.perm_tokens + first_draw, w13,
-            scratch.chunk_hidden, batch_count, widest, scratch.intermediate, scratch.hidden,
-            swiglu_limit, input_stride, stream);
+            batch_input, device_bounds, scratch.perm_tokens, gate_up, scratch.chunk_hidden, in_window,
+            widest, scratch.intermediate, scratch.hidden, swiglu_limit, input_stride, stream);
         kernel::dispatch_aeon_moe_grouped_w2_wmma<4, 8, 4, kernel::kMoeGroupedMTiles>(
-            scratch.chunk_hidden, scratch.batch_offsets, scratch.perm_draws + first_draw,
-            scratch.perm_weights + first_draw, w2, scratch.chunk_contrib, batch_count, widest,
-            scratch.hidden, scratch.intermediate, stream);
+            scratch.chunk_hidden, device_bounds, scratch.perm_draws, scratch.perm_weights, down,
+            scratch.chunk_contrib, in_window, widest, scratch.hidden, scratch.intermediate, stream);
     }
 
-    constexpr int kThreads = 256;
-    for (uint32_t token = 0; token < token_count; ++token) {
-        half* accum = batch_output + static_cast<size_t>(token) * output_stride;
-        kernel::moe_accumulate_fixed_order_kernel<<<(scratch.hidden + kThreads - 1) / kThreads,
-                                                    kThreads, 0, stream>>>(
-            scratch.chunk_contrib + static_cast<size_t>(token) * slots * scratch.hidden, slots, accum,
-            accum, scratch.hidden);
-    }
+    aeon355::throw_on_error(aeon_moe_accumulate_fixed_order_tokens(
+        scratch.chunk_contrib, tokens, slots, batch_output, output_stride, scratch.hidden, stream));
 }
 
 }  // namespace aeon::core
