@@ -43,7 +43,7 @@ struct ExpertFormatDescriptor {
         const bool sector_ok = sector_size > 0 && (sector_size & (sector_size - 1)) == 0;
         expert_format_detail::require(
             sector_ok && payload_bytes > 0 && payload_bytes % sector_size == 0,
-            "ExpertFormatDescriptor: payload must be a non-zero multiple of sector_size");
+            "expert format: payload_bytes is not a positive whole number of power-of-two sectors");
     }
 
     // On top of that a catalog names at least one expert, and few enough for a 16-byte index
@@ -53,7 +53,7 @@ struct ExpertFormatDescriptor {
         expert_format_detail::require(
             num_layers > 0 && experts_per_layer > 0 &&
                 total_experts() <= std::numeric_limits<size_t>::max() / 16,
-            "ExpertFormatDescriptor: layer and expert counts must describe a valid catalog");
+            "expert format: a catalog needs at least one layer and one expert per layer, and an index that fits");
     }
 };
 
