@@ -41,8 +41,37 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int* wave_totals, int
 }
 
 // A batch of at most this many draws is scattered by the workgroup that counts it (one launch
-// instead of two: a decode step is short enough for a launch to show).
+// instead of two: a decode step is short enough for a launch to show). Larger batches are
+// scattered in chunks of this many draws, one workgroup each.
 constexpr int kFusedScatterDraws = 1024;
+constexpr int kWaveCountWords = (kFusedScatterDraws / 64) * (kMaxPermutationExperts + 1) / 2 + 1;
+
+// Stable rank of each of a 1024-thread workgroup's draws among the workgroup's draws of the same
+// expert: thread i holds draw i of the chunk (`mine` = its expert, -1 for none), wave w the draws
+// 64w..64w+63. The earlier waves' share comes from per-wave counts in LDS (`wave_count`, zeroed
+// here), the share of the lower lanes from a walk over the wave's own 64 draws. Ends with the
+// workgroup synchronised.
+__device__ __forceinline__ int rank_in_chunk(int mine, int lists, uint32_t* wave_count_words) {
+    unsigned short* wave_count = reinterpret_cast<unsigned short*>(wave_count_words);
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < (16 * lists + 1) / 2; i += blockDim.x) wave_count_words[i] = 0;
+    __syncthreads();
+    int rank = 0, later = 0;
+#pragma unroll 8
+    for (int l = 0; l < 64; ++l) {
+        const bool same = __builtin_amdgcn_readlane(mine, l) == mine;
+        rank += (l < lane && same) ? 1 : 0;
+        later += (l > lane && same) ? 1 : 0;
+    }
+    // the last lane of an expert in the wave knows the wave's count for it
+    if (mine >= 0 && later == 0) wave_count[wave * lists + mine] = static_cast<unsigned short>(rank + 1);
+    __syncthreads();
+    if (mine >= 0) {
+        for (int w = 0; w < wave; ++w) rank += wave_count[w * lists + mine];
+    }
+    return rank;
+}
 
 template <bool SCATTER>
 __global__ __launch_bounds__(1024) void permutation_offsets_kernel(PermutationArgs a) {
@@ -94,31 +123,14 @@ __global__ __launch_bounds__(1024) void permutation_offsets_kernel(PermutationAr
 
     if (SCATTER) {
         // Draw d goes to its list's offset plus the number of earlier draws of the same expert
-        // (ascending draw order inside a list). Wave w holds draws 64w..64w+63: the earlier
-        // waves' share comes from per-wave counts in LDS, the share of the lower lanes from a
-        // walk over the wave's own 64 draws.
-        __shared__ uint32_t wave_count_words[(kFusedScatterDraws / 64) * (kMaxPermutationExperts + 1) / 2 + 1];
-        unsigned short* wave_count = reinterpret_cast<unsigned short*>(wave_count_words);
-        const int lane = threadIdx.x & 63;
-        const int wave = threadIdx.x >> 6;
-        const int waves = (a.draws + 63) / 64;
-        for (int i = threadIdx.x; i < (waves * lists + 1) / 2; i += blockDim.x) wave_count_words[i] = 0;
+        // (ascending draw order inside a list).
+        __shared__ uint32_t wave_count_words[kWaveCountWords];
         __syncthreads();
         if (e < lists) histogram[e] = offset;
         const int d = threadIdx.x;
         const int mine = d < a.draws ? draw_expert[d] : -1;
-        int rank = 0, later = 0;
-#pragma unroll 8
-        for (int l = 0; l < 64; ++l) {
-            const bool same = __builtin_amdgcn_readlane(mine, l) == mine;
-            rank += (l < lane && same) ? 1 : 0;
-            later += (l > lane && same) ? 1 : 0;
-        }
-        // the last lane of an expert in the wave knows the wave's count for it
-        if (mine >= 0 && later == 0) wave_count[wave * lists + mine] = static_cast<unsigned short>(rank + 1);
-        __syncthreads();
+        const int rank = rank_in_chunk(mine, lists, wave_count_words);
         if (mine >= 0) {
-            for (int w = 0; w < wave; ++w) rank += wave_count[w * lists + mine];
             const int at = histogram[mine] + rank;
             a.token_indices[at] = d / a.slots;
             a.draw_indices[at] = d;
@@ -135,57 +147,46 @@ __global__ __launch_bounds__(1024) void permutation_offsets_kernel(PermutationAr
     }
 }
 
-// One wave per expert list; the list past the routed experts is the always-on expert, which
-// takes every token once, in token order, with weight 1 and its own output rows.
-__global__ __launch_bounds__(256) void permutation_scatter_kernel(PermutationArgs a) {
-    const int lane = threadIdx.x & 63;
-    const int e = blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int lists = a.experts + (a.shared_tokens > 0 ? 1 : 0);
-    if (e >= lists) return;
-    int position = a.offsets[e];
-    const int end = a.offsets[e + 1];
-    if (position == end) return;
-    if (e == a.experts) {
-        for (int t = lane; t < a.shared_tokens; t += 64) {
-            a.token_indices[position + t] = t;
-            a.draw_indices[position + t] = a.draws + t;
-            if (a.weights_by_position != nullptr) a.weights_by_position[position + t] = 1.0f;
+// Scatter of a large batch: workgroup c places draws 1024c..1024c+1023. A draw goes to its
+// list's offset + the draws of the same expert in earlier chunks (counted here from the ids, an
+// LDS histogram: counts do not depend on the order of the adds) + its stable rank inside the
+// chunk. The workgroups past the last chunk write the always-on expert's list, which takes
+// every token once, in token order, with weight 1 and its own output rows.
+__global__ __launch_bounds__(1024) void permutation_scatter_kernel(PermutationArgs a) {
+    __shared__ int before[kMaxPermutationExperts + 1];
+    __shared__ uint32_t wave_count_words[kWaveCountWords];
+    const int chunks = (a.draws + kFusedScatterDraws - 1) / kFusedScatterDraws;
+    const int chunk = blockIdx.x;
+    if (chunk >= chunks) {
+        const int base = a.offsets[a.experts];
+        for (int t = (chunk - chunks) * blockDim.x + threadIdx.x; t < a.shared_tokens;
+             t += (gridDim.x - chunks) * blockDim.x) {
+            a.token_indices[base + t] = t;
+            a.draw_indices[base + t] = a.draws + t;
+            if (a.weights_by_position != nullptr) a.weights_by_position[base + t] = 1.0f;
         }
         return;
     }
-    // The scan is a chain of loads whose results decide nothing about the next address, so
-    // 32 rounds of ids are requested together: the wave pays one memory latency per 2048
-    // draws instead of one per 64.
-    constexpr int kRounds = 32;
-    // token = draw / slots without the emulated integer division (it dominated the scan): the
-    // product with ceil(2^32 / slots) is exact while draw * slots < 2^32, which the launcher
-    // checks before choosing this form.
-    const unsigned magic = a.slots_reciprocal;
-    for (int base = 0; base < a.draws && position < end; base += 64 * kRounds) {
-        int id[kRounds];
-        float weight[kRounds];
-#pragma unroll
-        for (int j = 0; j < kRounds; ++j) {
-            const int d = base + j * 64 + lane;
-            id[j] = d < a.draws ? a.ids[d] : -1;
-            // fetched with the ids, not inside the branch below: a load there would stall the
-            // wave for a memory latency in every round that places anything
-            weight[j] = d < a.draws && a.weights_by_draw != nullptr ? a.weights_by_draw[d] : 0.0f;
-        }
-#pragma unroll
-        for (int j = 0; j < kRounds; ++j) {
-            const int d = base + j * 64 + lane;
-            const bool mine = id[j] == e;
-            const unsigned long long mask = __ballot(mine);
-            if (mine) {
-                const int at = position + __popcll(mask & ((1ull << lane) - 1ull));
-                a.token_indices[at] = magic != 0 ? static_cast<int>(__umulhi(static_cast<unsigned>(d), magic))
-                                                 : d / a.slots;
-                a.draw_indices[at] = d;
-                if (a.weights_by_position != nullptr) a.weights_by_position[at] = weight[j];
-            }
-            position += __popcll(mask);
-        }
+    const int lists = a.experts + (a.shared_tokens > 0 ? 1 : 0);
+    for (int e = threadIdx.x; e < lists; e += blockDim.x) before[e] = 0;
+    __syncthreads();
+    const int first = chunk * kFusedScatterDraws;
+    for (int d = threadIdx.x; d < first; d += blockDim.x) {
+        const int e = a.ids[d];
+        if (e >= 0 && e < a.experts) atomicAdd(&before[e], 1);
+    }
+    const int d = first + threadIdx.x;
+    int mine = d < a.draws ? a.ids[d] : -1;
+    if (mine < 0 || mine >= a.experts) mine = -1;  // out-of-range ids are dropped, not trusted
+    const float weight = mine >= 0 && a.weights_by_draw != nullptr ? a.weights_by_draw[d] : 0.0f;
+    const int rank = rank_in_chunk(mine, lists, wave_count_words);  // synchronises: `before` is complete
+    if (mine >= 0) {
+        const int at = a.offsets[mine] + before[mine] + rank;
+        a.token_indices[at] = a.slots_reciprocal != 0
+                                  ? static_cast<int>(__umulhi(static_cast<unsigned>(d), a.slots_reciprocal))
+                                  : d / a.slots;
+        a.draw_indices[at] = d;
+        if (a.weights_by_position != nullptr) a.weights_by_position[at] = weight;
     }
 }
 
@@ -202,8 +203,9 @@ int launch_permutation(const PermutationArgs& args, hipStream_t stream) {
     }
     permutation_offsets_kernel<false><<<1, 1024, 0, stream>>>(a);
     AEON_LAUNCH_CHECK();
-    const int lists = a.experts + (a.shared_tokens > 0 ? 1 : 0);
-    permutation_scatter_kernel<<<(lists + 3) / 4, 256, 0, stream>>>(a);
+    const int chunks = (a.draws + kFusedScatterDraws - 1) / kFusedScatterDraws;
+    const int shared_groups = a.shared_tokens > 0 ? (a.shared_tokens + 4095) / 4096 : 0;
+    permutation_scatter_kernel<<<chunks + shared_groups, 1024, 0, stream>>>(a);
     AEON_LAUNCH_CHECK();
     return AEON_OK;
 }
