@@ -101,7 +101,8 @@ def test_router_ids_bit_exact_on_identical_logits(orc, score_kind, k, scaling):
 
 @pytest.mark.parametrize("T,slots,E", [(1, 8, 256), (7, 6, 256), (300, 6, 256), (64, 8, 8),
                                        (0, 8, 256), (2048, 8, 256), (64, 8, 1024),
-                                       (128, 8, 256), (129, 8, 256), (1024, 1, 3), (171, 6, 1024)])
+                                       (128, 8, 256), (129, 8, 256), (1024, 1, 3), (171, 6, 1024),
+                                       (8192, 8, 256), (5000, 3, 1000)])
 def test_expert_permutation_bit_exact(orc, T, slots, E):
     """Cases of tests/test_expert_permutation.cpp (T=1,7,300,64 at E=8, 0) plus the prefill size
     and the sizes either side of 1024 draws, where the one-launch form hands over to the
