@@ -5,9 +5,10 @@
 // offsets[e] .. offsets[e+1); inside an expert the draws appear in ascending draw index, so the
 // placement is a pure function of the ids; an id outside [0, experts) is dropped.
 // Histogram + scan run in one workgroup (LDS atomics on integers, so the totals do not depend
-// on arrival order). The scatter gives every expert its own wave, which walks the draws in
-// order with ballot/popcount prefix sums: parallel across experts, sequential inside one, and
-// therefore deterministic without the O(experts x draws) single-thread walk.
+// on arrival order). The placement of a draw is its list's offset + the number of earlier draws
+// of the same expert, found per chunk of 1024 draws (per-wave counts + a walk over the wave's
+// own 64 draws) plus, for later chunks, a count of the chunks before: parallel over the draws,
+// deterministic, and without the O(experts x draws) single-thread walk.
 #include "permutation.hpp"
 
 namespace aeon355 {
