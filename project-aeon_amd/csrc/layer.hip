@@ -158,6 +158,14 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
                            (layer->hidden / 16) % (4 * rows_down) == 0;
     p.seg_tokens = grouped ? kGroupedTokensPerTile : both_wide ? kWideSegTokens : kSegTokens;
     p.seg_capacity = grouped ? lists + w.positions / kGroupedTokensPerTile + 1 : w.seg_capacity;
+    if (grouped) {
+        // the grouped kernels address activation rows with 32-bit byte offsets from one base
+        AEON_REQUIRE(static_cast<size_t>(tokens) * x_stride * 2 < (size_t{1} << 32) &&
+                         static_cast<size_t>(w.positions) * layer->intermediate * 2 < (size_t{1} << 32),
+                     AEON_ERR_INVALID_ARGUMENT,
+                     "%s: a chunk of %d tokens at this shape exceeds the 4 GiB the grouped kernels "
+                     "address; split the chunk", who, tokens);
+    }
     if (stage_mask & AEON_STAGE_PERMUTATION) {
         if (int rc = launch_permutation(p, s)) return rc;
     }
