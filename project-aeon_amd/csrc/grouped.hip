@@ -9,9 +9,9 @@
 //     v_mfma_f32_16x16x32_f16 and multiplies by the row's fp16 scale (one rounding per weight,
 //     as the reference's grouped feed does); the fragment is then reused for every token tile
 //     of the window, which is what makes the dequantisation cheap next to the MFMAs;
-//   * the window's live count picks the body: 1, 2, 3 or 4 token tiles with a deep ring of K
-//     groups in flight (grouped_run: bound by the latency of the weight stream), or 6 or 8 in
-//     a hand-pipelined body (grouped_run_full: bound by arithmetic), so an expert with a
+//   * the window's live count picks the body: 1, 2, 3 or 4 token tiles with three K groups in
+//     flight (bound by the latency of the weight stream) or 6 or 8 with one (bound by
+//     arithmetic), all hand-pipelined block by block (grouped_run), so an expert with a
 //     handful of tokens costs its weight stream and little else and no window computes more
 //     than two token tiles of padding.
 // Weights are read once per (expert, position tile); tiles of one expert are adjacent in the
@@ -40,223 +40,34 @@ __device__ __forceinline__ half8_t scaled_fragment(uint32_t word, half2_t scale2
 // vmcnt in bits 3:0 and 15:14, the export and LDS/scalar counters left at "no wait").
 #define AEON_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | 0x0F70)
 
-// The body for a window of LIVE token tiles (LIVE is the tile's live count rounded up to a power
-// of two; rows past the count are clamped reads whose results are never stored), with the
-// weights and the activation window of DEPTH later K groups in flight while one is computed.
+// The body for a window of LIVE token tiles (rows past the tile's live count are clamped reads
+// whose results are never stored), with the weights and the activation window of DEPTH later K
+// groups in flight while one is computed: small windows are bound by the latency of the weight
+// stream and keep three groups in flight in the registers and LDS their few accumulators leave
+// free, wide ones are bound by arithmetic and keep one.
 //
-// Windows with few tokens are bound by the latency of the weight stream, not by arithmetic: they
-// have few accumulators, so the registers (and the LDS a small window leaves free) go into a deep
-// ring instead. A full window is MFMA-bound, re-reads weights its neighbour tiles have just
-// pulled into L2, and keeps one group in flight.
-//
-// Inside a K step everything is straight-line code: the B fragments of an MFMA step are requested
-// together and the next step's weight fragments are unpacked while the current step's MFMAs run.
-// Loads complete in issue order and every K step issues the same number, so "the window of the
-// next group has landed" is a bound on the count of outstanding loads. The step ends in a bare
-// s_barrier: a wave arrives only after its own window requests have landed in LDS and after it
-// has consumed its reads of the slot about to be overwritten, which is all the ordering the
-// ring needs (the fences of __syncthreads would drain the whole ring every step).
-template <bool GATE_UP, int R, int LIVE, int DEPTH>
-__device__ __forceinline__ void grouped_run(const SegGateUpArgs& gu, const SegDownArgs& dn,
-                                            const aeon_a64_expert& e, int first, int count,
-                                            half8_t* xs_flat) {
-    constexpr int NM = GATE_UP ? 2 : 1;
-    constexpr int STAGES = DEPTH + 1;
-    constexpr int kBufferStride = LIVE * 4 * 64;  // in 16-byte units
-    constexpr int kLoadsPerStep = LIVE + NM * R * 2;
-    constexpr int kInFlight = (DEPTH - 1) * kLoadsPerStep;
-    static_assert(STAGES * LIVE <= 2 * kGroupedMT, "ring must fit the window buffer");
-    static_assert(kInFlight < 64, "vmcnt is a 6-bit counter");
-    constexpr bool kOverlapUnpack = true;
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int n = lane & 15;
-    const int chunk = lane >> 4;
-    const int tile0 = (blockIdx.x * 4 + wave) * R;
-
-    const int K = GATE_UP ? gu.H : dn.I;
-    const int groups = K / 128;
-    // Uniform base + 32-bit lane offset addressing keeps the address registers few.
-    const AEON_GLOBAL char* pm[NM];
-    const AEON_GLOBAL char* sm[NM];
-    pm[0] = as_global<char>(GATE_UP ? e.w1_packed : e.w2_packed);
-    sm[0] = as_global<char>(GATE_UP ? e.w1_scale : e.w2_scale);
-    if (GATE_UP) {
-        pm[NM - 1] = as_global<char>(e.w3_packed);
-        sm[NM - 1] = as_global<char>(e.w3_scale);
-    }
-    uint32_t woff[R], soff[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const uint32_t t = static_cast<uint32_t>(tile0 + r) * groups;
-        woff[r] = (t * 64 + lane) * 16;
-        soff[r] = (t * 16 + n) * 2;  // the A operand's row is lane % 16
-    }
-
-    // Staging: the window is LIVE*4 fragments of 1 KiB (token tile j, MFMA step st); wave w
-    // stages step w of every token tile. Lane (n, chunk) of a fragment fetches 16 bytes of row
-    // j*16+n at column w*32 + chunk*8 straight into its own 16-byte slot of the fragment
-    // (global_load_lds), which is the exact image the B-operand read wants.
-    const AEON_GLOBAL char* xbase = as_global<char>(GATE_UP ? static_cast<const void*>(gu.x)
-                                                            : static_cast<const void*>(dn.hidden));
-    uint32_t xoff[LIVE];
-#pragma unroll
-    for (int j = 0; j < LIVE; ++j) {
-        const int row = j * 16 + n;
-        const int live_row = row < count ? row : count - 1;
-        const int position = first + live_row;
-        const int column = wave * 32 + chunk * 8;
-        if (GATE_UP) {
-            const long src_row = gu.row_index != nullptr ? gu.row_index[position] : position;
-            xoff[j] = static_cast<uint32_t>((src_row * gu.x_stride + column) * 2);
-        } else {
-            xoff[j] = static_cast<uint32_t>((static_cast<size_t>(position) * dn.I + column) * 2);
-        }
-    }
-
-    float4_t acc[NM][R][LIVE];
-#pragma unroll
-    for (int m = 0; m < NM; ++m)
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int mt = 0; mt < LIVE; ++mt) acc[m][r][mt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-
-    u32x4_t wq[STAGES][NM][R];
-    uint16_t sc[STAGES][NM][R];
-
-    // Requests for K group g (clamped to the last one so every step issues the same count; the
-    // clamped repeats land in ring slots nobody reads again).
-#define AEON_GROUPED_ISSUE(g_, stage_)                                                              \
-    do {                                                                                            \
-        const int gi_ = (g_) < groups ? (g_) : groups - 1;                                          \
-        _Pragma("unroll") for (int j = 0; j < LIVE; ++j) {                                          \
-            __builtin_amdgcn_global_load_lds(                                                       \
-                (const AEON_GLOBAL void*)(xbase + (xoff[j] + static_cast<uint32_t>(gi_) * 256u)),   \
-                (__attribute__((address_space(3))) void*)(xs_flat + (stage_) * kBufferStride +      \
-                                                          (j * 4 + wave) * 64),                     \
-                16, 0, 0);                                                                          \
-        }                                                                                           \
-        _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                            \
-            _Pragma("unroll") for (int r = 0; r < R; ++r) {                                         \
-                wq[stage_][m][r] = *(const AEON_GLOBAL u32x4_t*)(                                   \
-                    pm[m] + (woff[r] + static_cast<uint32_t>(gi_) * 1024u));                        \
-                sc[stage_][m][r] = *(const AEON_GLOBAL uint16_t*)(                                  \
-                    sm[m] + (soff[r] + static_cast<uint32_t>(gi_) * 32u));                          \
-            }                                                                                       \
-        }                                                                                           \
-    } while (0)
-
-#pragma unroll
-    for (int s = 0; s < DEPTH; ++s) AEON_GROUPED_ISSUE(s, s);
-    AEON_WAIT_VMCNT(kInFlight);
-    __builtin_amdgcn_s_barrier();
-
-    for (int g0 = 0; g0 < groups; g0 += STAGES) {
-#pragma unroll
-        for (int s = 0; s < STAGES; ++s) {
-            const int g = g0 + s;
-            if (g < groups) {
-                AEON_GROUPED_ISSUE(g + DEPTH, (s + DEPTH) % STAGES);
-                half2_t scur[NM][R];
-#pragma unroll
-                for (int m = 0; m < NM; ++m)
-#pragma unroll
-                    for (int r = 0; r < R; ++r) {
-                        union { uint16_t u; half_t h; } v;
-                        v.u = sc[s][m][r];
-                        scur[m][r] = half2_t{v.h, v.h};
-                    }
-                const half8_t* xb = xs_flat + s * kBufferStride;
-                half8_t a[NM][R];
-#pragma unroll
-                for (int m = 0; m < NM; ++m)
-#pragma unroll
-                    for (int r = 0; r < R; ++r) a[m][r] = scaled_fragment(wq[s][m][r][0], scur[m][r]);
-#pragma unroll
-                for (int st = 0; st < 4; ++st) {
-                    half8_t b[LIVE];
-#pragma unroll
-                    for (int mt = 0; mt < LIVE; ++mt) b[mt] = xb[(mt * 4 + st) * 64 + lane];
-                    half8_t a_next[NM][R];
-                    if (kOverlapUnpack && st < 3) {
-#pragma unroll
-                        for (int m = 0; m < NM; ++m)
-#pragma unroll
-                            for (int r = 0; r < R; ++r)
-                                a_next[m][r] = scaled_fragment(wq[s][m][r][st < 3 ? st + 1 : 3], scur[m][r]);
-                    }
-#pragma unroll
-                    for (int mt = 0; mt < LIVE; ++mt)
-#pragma unroll
-                        for (int m = 0; m < NM; ++m)
-#pragma unroll
-                            for (int r = 0; r < R; ++r)
-                                acc[m][r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                    a[m][r], b[mt], acc[m][r][mt], 0, 0, 0);
-                    if (st < 3) {
-#pragma unroll
-                        for (int m = 0; m < NM; ++m)
-#pragma unroll
-                            for (int r = 0; r < R; ++r)
-                                a[m][r] = kOverlapUnpack
-                                              ? a_next[m][r]
-                                              : scaled_fragment(wq[s][m][r][st < 3 ? st + 1 : 3], scur[m][r]);
-                    }
-                }
-                AEON_WAIT_VMCNT(kInFlight);
-                __builtin_amdgcn_s_barrier();
-            }
-        }
-    }
-#undef AEON_GROUPED_ISSUE
-
-#pragma unroll
-    for (int mt = 0; mt < LIVE; ++mt) {
-        const int row = mt * 16 + n;  // position within the tile
-        if (row < count) {
-            const int position = first + row;
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const int row0 = (tile0 + r) * 16 + chunk * 4;
-                if (GATE_UP) {
-                    const float4_t& ga = acc[0][r][mt];
-                    const float4_t& up = acc[NM - 1][r][mt];
-                    uint2 packed;
-                    packed.x = float_to_half_bits(clamped_swiglu(ga[0], up[0], gu.limit)) |
-                               (static_cast<uint32_t>(float_to_half_bits(
-                                    clamped_swiglu(ga[1], up[1], gu.limit))) << 16);
-                    packed.y = float_to_half_bits(clamped_swiglu(ga[2], up[2], gu.limit)) |
-                               (static_cast<uint32_t>(float_to_half_bits(
-                                    clamped_swiglu(ga[3], up[3], gu.limit))) << 16);
-                    *reinterpret_cast<uint2*>(gu.hidden + static_cast<size_t>(position) * gu.I + row0) = packed;
-                } else {
-                    const float w = dn.weight[position];
-                    const float4_t& a4 = acc[0][r][mt];
-                    const float4_t v = {w * a4[0], w * a4[1], w * a4[2], w * a4[3]};
-                    const size_t out_row = dn.out_row != nullptr ? dn.out_row[position] : position;
-                    *reinterpret_cast<float4_t*>(dn.contrib + out_row * dn.H + row0) = v;
-                }
-            }
-        }
-    }
-}
-
-// The body for a wide window (six or eight token tiles), where arithmetic bounds the time. A K
-// group is 4*LIVE blocks; block (st, mt) is the NM*R MFMAs of MFMA step st on token tile mt. VALU work hides
-// behind the matrix pipe only when the same wave issues it right after an MFMA, so the group is
-// software-pipelined by hand, block by block:
+// A K group is 4*LIVE blocks; block (st, mt) is the NM*R MFMAs of MFMA step st on token tile mt.
+// VALU work hides behind the matrix pipe only when the same wave issues it right after an MFMA,
+// so the group is software-pipelined by hand, block by block:
 //   * the B fragments of a pair of blocks are read from LDS one pair early;
 //   * the weight fragments of MFMA step st+1 (for st = 3: step 0 of the next K group) are
-//     unpacked one fragment per two blocks, behind the MFMAs of step st;
-//   * a scheduling fence after every block keeps the compiler from regrouping any of it.
-// One K group of weights and activations is in flight while one is computed (two ring slots).
-template <bool GATE_UP, int R, int LIVE>
-__device__ __forceinline__ void grouped_run_full(const SegGateUpArgs& gu, const SegDownArgs& dn,
+//     unpacked in shares spread over the blocks of step st, behind their MFMAs;
+//   * the fragment registers alternate by step parity, so nothing is copied;
+//   * a scheduling fence after every pair keeps the compiler from regrouping any of it.
+// Loads complete in issue order and every group issues the same number, so "group g+1 has
+// landed" is a bound on the count of outstanding loads; a group ends in a bare s_barrier (the
+// fences of __syncthreads would wait for every LDS-DMA request and drain the ring).
+template <bool GATE_UP, int R, int LIVE, int DEPTH>
+__device__ __forceinline__ void grouped_run(const SegGateUpArgs& gu, const SegDownArgs& dn,
                                                  const aeon_a64_expert& e, int first, int count,
                                                  half8_t* xs_flat) {
-    static_assert(LIVE % 2 == 0 && LIVE <= kGroupedMT, "blocks go in pairs");
+    static_assert(LIVE >= 1 && LIVE <= kGroupedMT, "a window holds at most kGroupedMT token tiles");
     constexpr int NM = GATE_UP ? 2 : 1;
+    constexpr int STAGES = DEPTH + 1;
+    constexpr int kLoadsPerGroup = LIVE + NM * R * 2;
+    static_assert(STAGES * LIVE <= 2 * kGroupedMT, "the ring must fit the window buffer");
+    static_assert(STAGES >= 2 && STAGES <= 4, "the turn of the ring is written out for 2..4 slots");
+    static_assert((DEPTH - 1) * kLoadsPerGroup < 64, "vmcnt is a 6-bit counter");
     constexpr int kFrags = NM * R;
     constexpr int kBufferStride = LIVE * 4 * 64;  // in 16-byte units
     constexpr int kBlocks = 4 * LIVE;
@@ -309,8 +120,8 @@ __device__ __forceinline__ void grouped_run_full(const SegGateUpArgs& gu, const 
 #pragma unroll
             for (int mt = 0; mt < LIVE; ++mt) acc[m][r][mt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-    u32x4_t wq[2][NM][R];
-    uint16_t sc[2][NM][R];
+    u32x4_t wq[STAGES][NM][R];
+    uint16_t sc[STAGES][NM][R];
 #define AEON_FULL_ISSUE(g_, stage_)                                                                 \
     do {                                                                                            \
         const int gi_ = (g_) < groups ? (g_) : groups - 1;                                          \
@@ -341,8 +152,11 @@ __device__ __forceinline__ void grouped_run_full(const SegGateUpArgs& gu, const 
         return xs_flat[slot * kBufferStride + ((i % LIVE) * 4 + i / LIVE) * 64 + lane];
     };
 
-    AEON_FULL_ISSUE(0, 0);
-    AEON_WAIT_VMCNT(0);
+    // Loads complete in issue order and every group issues the same number, so "group g+1 has
+    // landed" is a bound on the number of younger requests still outstanding.
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) AEON_FULL_ISSUE(d, d);
+    AEON_WAIT_VMCNT((DEPTH - 1) * kLoadsPerGroup);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
 
@@ -358,54 +172,56 @@ __device__ __forceinline__ void grouped_run_full(const SegGateUpArgs& gu, const 
     b[1] = fragment(0, 1);
     __builtin_amdgcn_sched_barrier(0);
 
-    // One K group out of ring slot s; group g+1 is requested into the other slot first.
+    // One K group out of ring slot s; group g+DEPTH is requested first, into the slot the previous
+    // group was computed from (free since the barrier that ended it).
     // Blocks go in pairs. While LDS-DMA requests are outstanding the compiler waits for every
     // LDS read at once, so the two reads of the next pair are placed behind the first MFMA of
     // this pair -- behind the wait for this pair's own fragments -- and have the pair's eight
     // MFMAs to land.
     auto step = [&](int g, auto slot) {
         constexpr int s = decltype(slot)::value;
-        constexpr int sn = 1 - s;
-        AEON_FULL_ISSUE(g + 1, sn);
+        constexpr int sn = (s + 1) % STAGES;
+        AEON_FULL_ISSUE(g + DEPTH, (s + DEPTH) % STAGES);
         __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 0; i < kBlocks; i += 2) {
+        // the MFMAs of block i and this block's share of the next MFMA step's weight fragments
+        // (for the last step: of step 0 of the next K group, out of the next ring slot)
+        auto block = [&](int i, bool skip_first) {
             const int st = i / LIVE, mt = i % LIVE;
-            if (i == 3 * LIVE) {
-                // this wave's requests for group g+1 were made a whole group's arithmetic ago;
-                // its weights are unpacked from here on
-                AEON_WAIT_VMCNT(0);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            acc[0][0][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[st % 2][0][0], b[i % 4], acc[0][0][mt], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            if (i + 2 < kBlocks) {
-                b[(i + 2) % 4] = fragment(s, i + 2);
-                b[(i + 3) % 4] = fragment(s, i + 3);
-            }
 #pragma unroll
             for (int m = 0; m < NM; ++m)
 #pragma unroll
                 for (int r = 0; r < R; ++r)
-                    if (m + r > 0)
+                    if (!(skip_first && m + r == 0))
                         acc[m][r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[st % 2][m][r], b[i % 4],
                                                                                 acc[m][r][mt], 0, 0, 0);
 #pragma unroll
-            for (int m = 0; m < NM; ++m)
-#pragma unroll
-                for (int r = 0; r < R; ++r)
-                    acc[m][r][mt + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[st % 2][m][r], b[(i + 1) % 4],
-                                                                                acc[m][r][mt + 1], 0, 0, 0);
-            // this pair's share of the four fragments of the next MFMA step
-#pragma unroll
             for (int f = 0; f < kFrags; ++f) {
-                if (f * (LIVE / 2) / kFrags == mt / 2) {
+                if (f * LIVE / kFrags == mt) {
                     const int m = f / R, r = f % R;
                     a[(st + 1) % 2][m][r] =
                         st < 3 ? scaled_fragment(wq[s][m][r][st < 3 ? st + 1 : 0], scale_pair(sc[s][m][r]))
                                : scaled_fragment(wq[sn][m][r][0], scale_pair(sc[sn][m][r]));
                 }
             }
+        };
+#pragma unroll
+        for (int i = 0; i < kBlocks; i += 2) {
+            if (i <= 3 * LIVE && 3 * LIVE < i + 2) {
+                // the pair that starts the last MFMA step: from here on the weights of group
+                // g+1 are unpacked, and this wave's requests for them are at least two thirds of
+                // a group's arithmetic old
+                AEON_WAIT_VMCNT((DEPTH - 1) * kLoadsPerGroup);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            acc[0][0][i % LIVE] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                a[(i / LIVE) % 2][0][0], b[i % 4], acc[0][0][i % LIVE], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i + 2 < kBlocks) {
+                b[(i + 2) % 4] = fragment(s, i + 2);
+                b[(i + 3) % 4] = fragment(s, i + 3);
+            }
+            block(i, true);
+            block(i + 1, false);
             __builtin_amdgcn_sched_barrier(0);
         }
         // every wave's window of group g+1 has landed, and nobody reads slot s any more
@@ -415,12 +231,19 @@ __device__ __forceinline__ void grouped_run_full(const SegGateUpArgs& gu, const 
         b[1] = fragment(sn, 1);
         __builtin_amdgcn_sched_barrier(0);
     };
+    // whole turns of the ring as straight-line code, then the last partial turn
     int g = 0;
-    for (; g + 2 <= groups; g += 2) {
+    for (; g + STAGES <= groups; g += STAGES) {
         step(g, std::integral_constant<int, 0>{});
         step(g + 1, std::integral_constant<int, 1>{});
+        if constexpr (STAGES > 2) step(g + 2, std::integral_constant<int, 2>{});
+        if constexpr (STAGES > 3) step(g + 3, std::integral_constant<int, 3>{});
     }
     if (g < groups) step(g, std::integral_constant<int, 0>{});
+    if (g + 1 < groups) step(g + 1, std::integral_constant<int, 1>{});
+    if constexpr (STAGES > 3) {
+        if (g + 2 < groups) step(g + 2, std::integral_constant<int, 2>{});
+    }
 #undef AEON_FULL_ISSUE
 
 #pragma unroll
@@ -471,9 +294,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     const int live_tiles = (count + 15) >> 4;
     if (live_tiles > 6) {
-        grouped_run_full<GATE_UP, R, 8>(gu, dn, e, first, count, xs);
+        grouped_run<GATE_UP, R, 8, 1>(gu, dn, e, first, count, xs);
     } else if (live_tiles > 4) {
-        grouped_run_full<GATE_UP, R, 6>(gu, dn, e, first, count, xs);
+        grouped_run<GATE_UP, R, 6, 1>(gu, dn, e, first, count, xs);
     } else if (live_tiles > 3) {
         grouped_run<GATE_UP, R, 4, 3>(gu, dn, e, first, count, xs);
     } else if (live_tiles > 2) {
