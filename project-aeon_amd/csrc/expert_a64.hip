@@ -431,8 +431,6 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
     // LDS image of a group's activations: [buffer][token tile][MFMA step][lane] x 16 bytes
     auto slot = [&](int buffer, int mt, int st) { return xs + ((buffer * kWideMaxTiles + mt) * 4 + st) * 64 + lane; };
 #pragma unroll
-    for (int d = 0; d < D; ++d) load_group(d, d < groups ? d : groups - 1);
-#pragma unroll
     for (int mt = 0; mt < MT; ++mt) *slot(0, mt, wave) = *reinterpret_cast<const AEON_GLOBAL half8_t*>(xrow[mt]);
     // This wave's activation fragments of the next D groups wait in registers, fetched as far
     // ahead as the weights: loads complete in issue order, so a fragment fetched only one group
@@ -442,10 +440,16 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
     auto load_x = [&](int g, int mt) {
         return *reinterpret_cast<const AEON_GLOBAL half8_t*>(xrow[mt] + (g < groups ? g : groups - 1) * 128);
     };
+    // The requests of the first D groups go out in the order the loop keeps them in (weights
+    // of group d, then the fragment of group d+1): the compiler's wait counts are static, so a
+    // different order here would be the one every pass through the loop has to wait for.
 #pragma unroll
-    for (int d = 0; d < D; ++d)
+    for (int d = 0; d < D; ++d) {
+        load_group(d, d < groups ? d : groups - 1);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) xr[(d + 1) % D][mt] = load_x(d + 1, mt);
+        __builtin_amdgcn_sched_barrier(0);
+    }
     __syncthreads();
 
     // step g: read all four fragments of group g from LDS, multiply, publish this wave's
@@ -459,27 +463,35 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int st = 0; st < 4; ++st) xf[mt][st] = *slot(g & 1, mt, st);
+        // The K steps run outermost and the wave's tiles innermost, so that consecutive matrix
+        // instructions belong to different accumulators: a chain of dependent ones would hold
+        // the SIMD for the latency of each.
+        float4_t t[NM][R][MT];
+#pragma unroll
+        for (int m = 0; m < NM; ++m)
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) t[m][r][mt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int st = 0; st < 4; ++st)
+#pragma unroll
+            for (int m = 0; m < NM; ++m)
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const half8_t a = unpack8_vec(wq[d][m][r][st]);
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        t[m][r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, xf[mt][st], t[m][r][mt], 0, 0, 0);
+                }
 #pragma unroll
         for (int m = 0; m < NM; ++m)
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 // scales of (tile, group): 16 rows x 2 bytes; this lane's rows are 4*chunk..+3
                 const u32x2_t sc = scale_rows[((m * R + r) * tile_u4 + g * 2) * 2];
-                if (MT == 1) {
-                    scale_add(acc[m][r][0], mfma_group(wq[d][m][r], xf[0]), sc);
-                } else {
-                    half8_t a[4];
 #pragma unroll
-                    for (int st = 0; st < 4; ++st) a[st] = unpack8_vec(wq[d][m][r][st]);
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) {
-                        float4_t t = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-                        for (int st = 0; st < 4; ++st)
-                            t = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[st], xf[mt][st], t, 0, 0, 0);
-                        scale_add(acc[m][r][mt], t, sc);
-                    }
-                }
+                for (int mt = 0; mt < MT; ++mt) scale_add(acc[m][r][mt], t[m][r][mt], sc);
             }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) *slot((g + 1) & 1, mt, wave) = xr[(d + 1) % D][mt];
