@@ -194,6 +194,48 @@ def test_config2_moe_layer_decode_reduced_experts(orc, B):
     assert np.array_equal(out2.cpu().numpy(), out)
 
 
+def test_config2_full_size_sampled(orc):
+    """BASELINE config 2 as written: batch 64, top-8 of 256 experts + the always-on one, fp32
+    router with sigmoid scores and bias, H=7168, I=2048. The oracle covers a sample of tokens
+    (ids bit-exact on the device's logits for all of them); the rest is covered by properties
+    that hold at any size: a token's output does not depend on the other tokens of the batch
+    (same bits under a reversed batch, same values to summation order when it is run alone
+    through the K-split kernels) and a second run gives the same bits."""
+    torch, h, capi, moe, synth = _setup()
+    H, I, E, k, B, limit = 7168, 2048, 256, 8, 64, 7.0
+    pool = moe.ExpertPool(E + 1, H, I)
+    assert pool.fill_synthetic(seed=0, first_expert_id=0) == 0
+    wr, bias = synth.router_weight(0, H, E), synth.router_bias(0, E)
+    layer = moe.MoeLayer(pool, E, k, True, limit, h.to_dev(wr), h.to_dev(bias), score_kind=1)
+    x = synth.activations(0, B, H, unit=1000 * B)
+    d_x = h.dev_half(x)
+    out_t, ids_t, w_t = layer.decode(d_x)
+    logits = layer.router_logits(d_x).cpu().numpy()
+    torch.cuda.synchronize()
+    out, ids, w = out_t.cpu().numpy(), ids_t.cpu().numpy(), w_t.cpu().numpy()
+    assert np.isfinite(out).all()
+    for t in range(B):
+        oi, ow = orc.router_topk(logits[t].astype(np.float64), bias.astype(np.float64), k, 1.0, 1)
+        assert np.array_equal(ids[t], oi)
+        assert np.abs(w[t] - ow).max() <= 1e-5
+    assert 60 <= np.unique(ids).size <= 140   # the biased router concentrates the routing
+    sample = [0, 31, 63]
+    needed = sorted(set(int(e) for t in sample for e in ids[t]))
+    experts = {e: h.Expert(0, e, H, I) for e in needed}
+    shared = h.Expert(0, E, H, I)
+    want = _oracle_layer(orc, h, experts, x[sample], ids[sample], w[sample], shared, limit)
+    assert np.abs(want).max() > 1.0
+    assert np.abs(out[sample] - want).max() <= 6e-3 * np.abs(want).max()
+    again, _, _ = layer.decode(d_x)
+    assert np.array_equal(again.cpu().numpy(), out)
+    rev = layer.routed(d_x.flip(0).contiguous(), ids_t.flip(0).contiguous(),
+                       w_t.flip(0).contiguous()).flip(0).cpu().numpy()
+    assert np.array_equal(rev, out)
+    for t in (5, 40):
+        alone = layer.routed(d_x[t:t + 1], ids_t[t:t + 1], w_t[t:t + 1]).cpu().numpy()
+        assert np.abs(alone[0] - out[t]).max() <= 1e-3 * np.abs(out[t]).max()
+
+
 @pytest.mark.parametrize("H,I,B", [(256, 128, 3), (256, 384, 5), (768, 256, 17), (256, 128, 70)])
 def test_layer_on_minimal_shapes(orc, H, I, B):
     """Shapes with fewer 128-column groups than a workgroup has K-split waves (a wave with no
