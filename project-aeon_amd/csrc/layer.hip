@@ -90,8 +90,15 @@ extern "C" int aeon_router_logits(const void*, int, const float*, float*, int, i
 extern "C" int aeon_moe_router(const float*, const float*, const int64_t*, const int32_t*, float*,
                                int32_t*, int, int, int, float, int, int, void*);
 
+// Positions (draws plus the always-on expert's tokens) are 32-bit indices everywhere below.
+static bool positions_fit(const aeon_moe_layer& L, int tokens) {
+    return static_cast<long long>(tokens) * (L.top_k + 1) < (1ll << 31);
+}
+
 extern "C" size_t aeon_moe_layer_workspace_bytes(const aeon_moe_layer* layer, int max_tokens) {
-    if (layer == nullptr || max_tokens <= 0) return 0;
+    if (layer == nullptr || max_tokens <= 0 || layer->top_k <= 0 || !positions_fit(*layer, max_tokens)) {
+        return 0;
+    }
     return carve(*layer, max_tokens, nullptr).bytes;
 }
 
@@ -108,6 +115,9 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
                  AEON_ERR_INVALID_ARGUMENT, "%s: bad token shape (tokens=%d x_stride=%d out_stride=%d)",
                  who, tokens, x_stride, out_stride);
     if (tokens == 0) return AEON_OK;
+    AEON_REQUIRE(positions_fit(*layer, tokens), AEON_ERR_INVALID_ARGUMENT,
+                 "%s: %d tokens x top-%d exceed 32-bit positions; split the chunk", who, tokens,
+                 layer->top_k);
     const LayerWorkspace w = carve(*layer, tokens, d_workspace);
     AEON_REQUIRE(workspace_bytes >= w.bytes, AEON_ERR_INVALID_ARGUMENT,
                  "%s: workspace of %zu bytes, %zu needed", who, workspace_bytes, w.bytes);
@@ -240,6 +250,9 @@ extern "C" int aeon_moe_layer_decode(const aeon_moe_layer* layer, const void* d_
     AEON_REQUIRE(tokens >= 0 && x_stride >= layer->hidden, AEON_ERR_INVALID_ARGUMENT,
                  "%s: bad token shape (tokens=%d x_stride=%d)", who, tokens, x_stride);
     if (tokens == 0) return AEON_OK;
+    AEON_REQUIRE(positions_fit(*layer, tokens), AEON_ERR_INVALID_ARGUMENT,
+                 "%s: %d tokens x top-%d exceed 32-bit positions; split the chunk", who, tokens,
+                 layer->top_k);
     const LayerWorkspace w = carve(*layer, tokens, d_workspace);
     AEON_REQUIRE(workspace_bytes >= w.bytes, AEON_ERR_INVALID_ARGUMENT,
                  "%s: workspace of %zu bytes, %zu needed", who, workspace_bytes, w.bytes);

@@ -223,7 +223,10 @@ extern "C" int aeon_expert_permutation(const int32_t* d_topk_indices, int token_
     const char* who = "aeon_expert_permutation";
     AEON_REQUIRE(d_topk_indices && d_expert_offsets && d_token_indices && d_draw_indices,
                  AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
-    AEON_REQUIRE(token_count >= 0 && slots > 0, AEON_ERR_INVALID_ARGUMENT, "%s: bad draw shape", who);
+    AEON_REQUIRE(token_count >= 0 && slots > 0 &&
+                     static_cast<long long>(token_count) * slots < (1ll << 31),
+                 AEON_ERR_INVALID_ARGUMENT, "%s: bad draw shape (tokens=%d slots=%d)", who,
+                 token_count, slots);
     AEON_REQUIRE(expert_count > 0 && expert_count <= kMaxPermutationExperts,
                  AEON_ERR_INVALID_ARGUMENT, "%s: expert count out of range", who);
     AEON_REQUIRE((d_weights_by_draw == nullptr) == (d_weights_by_position == nullptr),

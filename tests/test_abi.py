@@ -51,6 +51,8 @@ def test_argument_errors_without_device_work():
                   C.c_float(10.0), None)
     with pytest.raises(ValueError, match="expert count out of range"):
         capi.call("aeon_expert_permutation", one, 4, 6, 2000, one, one, one, None, None, None)
+    with pytest.raises(ValueError, match="bad draw shape"):
+        capi.call("aeon_expert_permutation", one, 1 << 29, 8, 256, one, one, one, None, None, None)
     with pytest.raises(ValueError, match="both a source and a destination"):
         capi.call("aeon_expert_permutation", one, 4, 6, 256, one, one, one, one, None, None)
     with pytest.raises(ValueError, match="wave64 packing"):
@@ -66,6 +68,13 @@ def test_argument_errors_without_device_work():
                   8, 4, None)
     with pytest.raises(ValueError, match="the sink holds"):
         capi.call("aeon_calibrate_mfma_f16", 1, 10, 4, one, C.c_size_t(512), None, None)
+    from project_aeon_amd import moe
+    cfg = moe.MoeLayerStruct(7168, 2048, 256, 8, 1, 7.0, 1, 1.0, 1, None, None, 16)
+    assert capi.lib().aeon_moe_layer_workspace_bytes(C.byref(cfg), 64) > 0
+    assert capi.lib().aeon_moe_layer_workspace_bytes(C.byref(cfg), 1 << 28) == 0
+    with pytest.raises(ValueError, match="32-bit positions"):
+        capi.call("aeon_moe_layer_routed", C.byref(cfg), one, 7168, 1 << 28, one, one, one, 7168, one,
+                  C.c_size_t(1 << 40), None)
     assert capi.lib().aeon_last_error() != b""
 
 
