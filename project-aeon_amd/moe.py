@@ -130,6 +130,11 @@ class MoeLayer:
             self.workspace_tokens = tokens
         return self.workspace
 
+    def _new_out(self, x):
+        # with an always-on expert every output row is overwritten; without one the routed sum
+        # is added to the row, which therefore has to start at zero
+        return torch.empty_like(x) if self.cfg.has_shared else torch.zeros_like(x)
+
     def decode(self, x, out=None, ids=None, weights=None):
         """x fp16 [tokens][hidden] -> (out fp16 [tokens][hidden], ids int32, weights fp32).
         Without an always-on expert the routed sum is added to what `out` holds, so an `out`
@@ -137,7 +142,7 @@ class MoeLayer:
         tokens = x.shape[0]
         ws = self._workspace(tokens)
         k = self.cfg.top_k
-        out = torch.zeros_like(x) if out is None else out
+        out = self._new_out(x) if out is None else out
         ids = torch.empty(tokens, k, dtype=torch.int32, device=x.device) if ids is None else ids
         weights = (torch.empty(tokens, k, dtype=torch.float32, device=x.device)
                    if weights is None else weights)
@@ -152,7 +157,7 @@ class MoeLayer:
         reference's in-place accumulator); an `out` allocated here therefore starts at zero."""
         tokens = x.shape[0]
         ws = self._workspace(tokens)
-        out = torch.zeros_like(x) if out is None else out
+        out = self._new_out(x) if out is None else out
         capi.call("aeon_moe_layer_routed", C.byref(self.cfg), capi.vp(x), x.stride(0), tokens,
                   capi.vp(ids), capi.vp(weights), capi.vp(out), out.stride(0), capi.vp(ws),
                   C.c_size_t(ws.numel()), stream_ptr())
@@ -267,15 +272,20 @@ class LayerStack:
         self.mixes = mixes
 
     def step(self, residual, scratch=None, trace=None):
-        """residual fp16 [4][tokens][hidden]; returns the new residual (a different buffer)."""
+        """residual fp16 [4][tokens][hidden]; returns the new residual (a different buffer).
+        `scratch` = (residual-shaped buffer, x [tokens][hidden]) and optionally the layer output,
+        ids and weights buffers every layer reuses."""
         streams, tokens, hidden = residual.shape
         if scratch is None:
             scratch = (torch.empty_like(residual), torch.empty(tokens, hidden, dtype=torch.float16,
                                                                device=residual.device))
-        other, x = scratch
+        other, x = scratch[:2]
+        bufs = scratch[2:] if len(scratch) > 2 else (None, None, None)
         for layer, hc in zip(self.layers, self.mixes):
             hc.pre_combine(residual, x)
-            y, ids, w = layer.decode(x)
+            if bufs[0] is not None and not layer.cfg.has_shared:
+                bufs[0].zero_()
+            y, ids, w = layer.decode(x, *bufs)
             hc.post_mix(y, residual, other)
             if trace is not None:
                 trace.append((residual.clone(), x.clone(), ids.clone(), w.clone(), y.clone(),
