@@ -266,7 +266,9 @@ size_t aeon_moe_layer_workspace_bytes(const aeon_moe_layer* layer, int max_token
  * given the routed ids/weights [tokens][top_k] on the device, out[t] = half(shared(x_t) as fp16
  * + sum_k w[t][k] * expert_{ids[t][k]}(x_t)) in slot order, fp32. Without a shared expert the
  * value already in d_out is the fp16 starting value, as moe_accum is in the reference. Each
- * distinct expert's weights are streamed once per 16 of its tokens. No host synchronisation. */
+ * distinct expert's weights are streamed once per 16 of its tokens. No host synchronisation.
+ * An id outside [0, experts) contributes nothing (the reference's permutation drops it,
+ * src/platform/ops/expert_permutation.hpp:64-70; here the reduce leaves its slot out as well). */
 int aeon_moe_layer_routed(const aeon_moe_layer* layer, const void* d_x, int x_stride, int tokens,
                           const int32_t* d_topk_ids, const float* d_topk_weights, void* d_out,
                           int out_stride, void* d_workspace, size_t workspace_bytes, void* stream);

@@ -634,9 +634,12 @@ int launch_seg_down(const SegDownArgs& a, int k_split, int row_tiles, int depth,
 // ---------------------------------------------------------------------------------------------
 
 // Four columns per thread (hidden is a multiple of 128): 16-byte loads of the fp32 contributions.
+// `ids` (may be null) are the token's expert choices: a slot whose id is outside [0, experts) was
+// dropped by the permutation, no kernel wrote its contribution row, and it is skipped here.
 __global__ __launch_bounds__(256) void token_reduce_kernel(
     const float* __restrict__ contrib, int slots, int shared_base, const uint16_t* initial,
-    long initial_stride, uint16_t* out, long out_stride, int hidden) {
+    long initial_stride, uint16_t* out, long out_stride, int hidden,
+    const int32_t* __restrict__ ids, int experts) {
     const int t = blockIdx.y;
     const int i = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (i >= hidden) return;
@@ -654,6 +657,10 @@ __global__ __launch_bounds__(256) void token_reduce_kernel(
     }
     const float* c = contrib + static_cast<size_t>(t) * slots * hidden + i;
     for (int s = 0; s < slots; ++s) {
+        if (ids != nullptr) {
+            const int e = ids[t * slots + s];
+            if (e < 0 || e >= experts) continue;
+        }
         const float4_t v = *reinterpret_cast<const float4_t*>(c + static_cast<size_t>(s) * hidden);
 #pragma unroll
         for (int q = 0; q < 4; ++q) acc[q] += v[q];
@@ -672,11 +679,12 @@ __global__ __launch_bounds__(256) void token_reduce_kernel(
 
 int launch_token_reduce(const float* contrib, int tokens, int slots, int shared_base,
                         const uint16_t* initial, long initial_stride, uint16_t* out,
-                        long out_stride, int hidden, hipStream_t stream) {
+                        long out_stride, int hidden, hipStream_t stream, const int32_t* ids,
+                        int experts) {
     if (tokens <= 0) return AEON_OK;
     AEON_REQUIRE(hidden % 4 == 0, AEON_ERR_INVALID_ARGUMENT, "token reduce: hidden %d is not a multiple of 4", hidden);
     token_reduce_kernel<<<dim3((hidden / 4 + 255) / 256, tokens), 256, 0, stream>>>(
-        contrib, slots, shared_base, initial, initial_stride, out, out_stride, hidden);
+        contrib, slots, shared_base, initial, initial_stride, out, out_stride, hidden, ids, experts);
     AEON_LAUNCH_CHECK();
     return AEON_OK;
 }

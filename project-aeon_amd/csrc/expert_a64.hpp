@@ -65,9 +65,11 @@ int launch_grouped_down(const SegDownArgs& a, hipStream_t stream);
 // out[t][i] = half( [shared: float(half(contrib[shared_base + t][i]))] +
 //                   sum_{s < slots, ascending} contrib[t*slots + s][i] ),
 // with `initial` (nullable, may alias out) added as the fp16 starting value when there is no
-// in-buffer shared row (shared_base < 0).
+// in-buffer shared row (shared_base < 0). With `ids` [tokens][slots] given, a slot whose id is
+// outside [0, experts) is left out of the sum (the permutation dropped it, so nothing wrote its row).
 int launch_token_reduce(const float* contrib, int tokens, int slots, int shared_base,
                         const uint16_t* initial, long initial_stride, uint16_t* out,
-                        long out_stride, int hidden, hipStream_t stream);
+                        long out_stride, int hidden, hipStream_t stream,
+                        const int32_t* ids = nullptr, int experts = 0);
 
 }  // namespace aeon355

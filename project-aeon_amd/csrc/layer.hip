@@ -215,7 +215,8 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     if (!(stage_mask & AEON_STAGE_REDUCE)) return AEON_OK;
     return launch_token_reduce(w.contrib, tokens, layer->top_k, layer->has_shared ? draws : -1,
                                layer->has_shared ? nullptr : static_cast<const uint16_t*>(d_out),
-                               out_stride, static_cast<uint16_t*>(d_out), out_stride, layer->hidden, s);
+                               out_stride, static_cast<uint16_t*>(d_out), out_stride, layer->hidden, s,
+                               d_topk_ids, layer->experts);
 }
 
 extern "C" int aeon_moe_layer_routed(const aeon_moe_layer* layer, const void* d_x, int x_stride,

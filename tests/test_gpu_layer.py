@@ -258,6 +258,38 @@ def test_layer_on_minimal_shapes(orc, H, I, B):
     assert np.abs(out - want).max() <= 6e-3 * np.abs(want).max()
 
 
+@pytest.mark.parametrize("T", [6, 150])
+def test_out_of_range_ids_contribute_nothing(orc, T):
+    """An id outside [0, experts) is dropped by the permutation (as the reference's does); the
+    slot-ordered reduce must then leave that slot out instead of adding a row nobody wrote. Run
+    on the decode (segment) path and on the grouped path, after a call that left other values in
+    the workspace."""
+    torch, h, capi, moe, synth = _setup()
+    H, I, E, k, limit = 256, 256, 12, 3, 7.0
+    pool = moe.ExpertPool(E + 1, H, I)
+    assert pool.fill_synthetic(seed=31, first_expert_id=0) == 0
+    layer = moe.MoeLayer(pool, E, k, True, limit)
+    rng = np.random.default_rng(31)
+    ids = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+    w = synth.route_weights(31, T * k).reshape(T, k).astype(np.float32)
+    x = synth.activations(31, T, H)
+    d_x = h.dev_half(x)
+    layer.routed(d_x, h.to_dev(ids), h.to_dev(w))          # fills every contribution row
+    bad = ids.copy()
+    bad[1, 0], bad[T - 1, k - 1], bad[2, 1] = -1, E, 1 << 20
+    out = layer.routed(d_x, h.to_dev(bad), h.to_dev(w)).cpu().numpy()
+    experts = {e: h.Expert(31, e, H, I) for e in range(E)}
+    shared = h.Expert(31, E, H, I)
+    check = [0, 1, 2, T - 1]
+    want = np.zeros((len(check), H))
+    for n, t in enumerate(check):
+        keep = [s for s in range(k) if 0 <= bad[t, s] < E]
+        row = _oracle_layer(orc, h, experts, x[t:t + 1], bad[t:t + 1, keep], w[t:t + 1, keep], shared, limit)
+        want[n] = row[0]
+    assert np.isfinite(out).all()
+    assert np.abs(out[check] - want).max() <= 6e-3 * np.abs(want).max()
+
+
 def test_decode_segments_of_two_token_tiles(orc):
     """A decode batch in which both launches take the wide form (many live experts) and single
     experts hold 40, 20, 17 and 16 positions: segments of 32+8, 20, 17 and 16 positions, i.e. the
