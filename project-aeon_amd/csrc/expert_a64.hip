@@ -200,11 +200,18 @@ __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegD
     int first = 0;
     int count = GATE_UP ? gu.direct_count : dn.direct_count;
     aeon_a64_expert e = GATE_UP ? gu.direct_expert : dn.direct_expert;
+    const bool slot_mode = seg.total == nullptr && seg.slot_experts > 0;
     if (seg.total != nullptr) {
         if (s >= *seg.total) return;
         first = seg.first[s];
         count = seg.count[s];
         e = (GATE_UP ? gu.experts : dn.experts)[seg.expert[s]];
+    } else if (slot_mode) {
+        const int id = s == seg.slot_shared ? seg.slot_experts : seg.expert[s];
+        if (id < 0 || (id >= seg.slot_experts && s != seg.slot_shared)) return;
+        first = s;
+        count = 1;
+        e = (GATE_UP ? gu.experts : dn.experts)[id];
     }
 
     const int lane = threadIdx.x & 63;
@@ -229,7 +236,7 @@ __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegD
     const int position = first + (n < count ? n : count - 1);
     const AEON_GLOBAL uint16_t* xrow;
     if (GATE_UP) {
-        const long row = gu.row_index != nullptr ? gu.row_index[position] : position;
+        const long row = slot_mode ? 0 : gu.row_index != nullptr ? gu.row_index[position] : position;
         xrow = as_global<uint16_t>(gu.x) + row * gu.x_stride + chunk * 8;
     } else {
         xrow = as_global<uint16_t>(dn.hidden) + static_cast<size_t>(position) * dn.I + chunk * 8;
@@ -334,7 +341,7 @@ __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegD
                             clamped_swiglu(ga[3], up[3], gu.limit))) << 16);
             *reinterpret_cast<uint2*>(gu.hidden + static_cast<size_t>(first + n) * gu.I + row0) = packed;
         } else {
-            const float w = dn.weight[first + n];
+            const float w = slot_mode && s == seg.slot_shared ? 1.0f : dn.weight[first + n];
             const float4_t v = {w * acc[0][r][0], w * acc[0][r][1], w * acc[0][r][2], w * acc[0][r][3]};
             const size_t out_row = dn.out_row != nullptr ? dn.out_row[first + n] : first + n;
             *reinterpret_cast<float4_t*>(dn.contrib + out_row * dn.H + row0) = v;
@@ -362,9 +369,12 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
                                               int row_block, half8_t* xs, u32x4_t* scale_lds) {
     constexpr int NM = GATE_UP ? 2 : 1;
     const SegmentList& seg = GATE_UP ? gu.seg : dn.seg;
-    const int first = seg.first[s];
-    const int count = seg.count[s];
-    const aeon_a64_expert e = (GATE_UP ? gu.experts : dn.experts)[seg.expert[s]];
+    // slot mode (single token, no segment list): segment s is slot s of the caller's ids
+    const bool slot_mode = seg.total == nullptr;
+    const int first = slot_mode ? s : seg.first[s];
+    const int count = slot_mode ? 1 : seg.count[s];
+    const int id = slot_mode && s == seg.slot_shared ? seg.slot_experts : seg.expert[s];
+    const aeon_a64_expert e = (GATE_UP ? gu.experts : dn.experts)[id];
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -391,7 +401,7 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
         const int token = mt * kSegTokens + n;
         const int position = first + (token < count ? token : count - 1);
         if (GATE_UP) {
-            const long row = gu.row_index != nullptr ? gu.row_index[position] : position;
+            const long row = slot_mode ? 0 : gu.row_index != nullptr ? gu.row_index[position] : position;
             xrow[mt] = as_global<uint16_t>(gu.x) + row * gu.x_stride + chunk * 8 + wave * 32;
         } else {
             xrow[mt] = as_global<uint16_t>(dn.hidden) + static_cast<size_t>(position) * dn.I + chunk * 8 +
@@ -535,7 +545,7 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
                                 clamped_swiglu(ga[3], up[3], gu.limit))) << 16);
                 *reinterpret_cast<uint2*>(gu.hidden + static_cast<size_t>(first + token) * gu.I + row0) = packed;
             } else {
-                const float w = dn.weight[first + token];
+                const float w = slot_mode && s == seg.slot_shared ? 1.0f : dn.weight[first + token];
                 const float4_t& a4 = acc[0][r][mt];
                 const float4_t v = {w * a4[0], w * a4[1], w * a4[2], w * a4[3]};
                 const size_t out_row = dn.out_row != nullptr ? dn.out_row[first + token] : first + token;
@@ -555,6 +565,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     extern __shared__ u32x4_t scale_lds[];  // [wave][m][r][groups * 2] 16-byte units
     const SegmentList& seg = GATE_UP ? gu.seg : dn.seg;
     const int s = blockIdx.y;  // the list is ordered costliest first
+    if (seg.total == nullptr) {
+        // slot mode: one token, segment s = slot s; a dropped id ends the workgroup
+        if (s != seg.slot_shared) {
+            const int id = seg.expert[s];
+            if (id < 0 || id >= seg.slot_experts) return;
+        }
+        seg_wide_item<GATE_UP, R, D, 1>(gu, dn, s, blockIdx.x, xs, scale_lds);
+        return;
+    }
     if (s >= *seg.total) return;
     if (seg.count[s] > kSegTokens) {
         seg_wide_item<GATE_UP, R, (D > 2 ? 2 : D), 2>(gu, dn, s, blockIdx.x, xs, scale_lds);
@@ -598,7 +617,8 @@ static void launch_seg_r(const SegGateUpArgs& gu, const SegDownArgs& dn, int til
 template <bool GATE_UP>
 static void launch_seg(const SegGateUpArgs& gu, const SegDownArgs& dn, int tiles, int capacity,
                        int k_split, int row_tiles, int depth, hipStream_t stream) {
-    const bool direct = (GATE_UP ? gu.seg.total : dn.seg.total) == nullptr;
+    const SegmentList& list = GATE_UP ? gu.seg : dn.seg;
+    const bool direct = list.total == nullptr && list.slot_experts == 0;
     if (k_split == 0 && (direct || tiles % (4 * (row_tiles >= 2 ? 2 : 1)) != 0)) {
         k_split = 1;  // the wide form needs a segment list and whole workgroups of tiles
     }

@@ -21,6 +21,12 @@ struct SegmentList {
     const int* total;   // [1] number of live segments (device); null = "direct" mode: one
                         // segment, positions 0..direct_count-1 of direct_expert
     int capacity;       // grid bound: blocks past *total exit at once
+    // "slot" mode for a single token (total == null, slot_experts > 0): segment s is the
+    // token's slot s -- expert[s] is read straight from the caller's top-k ids, position s,
+    // one token; an id outside [0, slot_experts) ends the workgroup. Segment `slot_shared`
+    // (if >= 0) is the always-on expert, table entry slot_experts, weight 1.
+    int slot_experts;
+    int slot_shared;
 };
 
 struct SegGateUpArgs {

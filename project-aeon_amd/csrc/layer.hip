@@ -176,7 +176,11 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
                      "%s: a chunk of %d tokens at this shape exceeds the 4 GiB the grouped kernels "
                      "address; split the chunk", who, tokens);
     }
-    if (stage_mask & AEON_STAGE_PERMUTATION) {
+    // A single token needs no permutation: slot s of its top-k is segment s, read by the
+    // kernels straight from the caller's ids and weights (the always-on expert, if any, is one
+    // more segment), and its contribution rows are already in draw order.
+    const bool slots_direct = tokens == 1;
+    if ((stage_mask & AEON_STAGE_PERMUTATION) && !slots_direct) {
         if (int rc = launch_permutation(p, s)) return rc;
     }
 
@@ -185,7 +189,13 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     gu.x_stride = x_stride;
     gu.row_index = w.token_indices;
     gu.experts = layer->d_experts;
-    gu.seg = SegmentList{w.seg_expert, w.seg_first, w.seg_count, w.seg_total, p.seg_capacity};
+    gu.seg = SegmentList{w.seg_expert, w.seg_first, w.seg_count, w.seg_total, p.seg_capacity, 0, -1};
+    if (slots_direct) {
+        gu.seg = SegmentList{d_topk_ids, nullptr, nullptr, nullptr,
+                             layer->top_k + (layer->has_shared ? 1 : 0), layer->experts,
+                             layer->has_shared ? layer->top_k : -1};
+        gu.row_index = nullptr;
+    }
     gu.hidden = w.hidden;
     gu.H = layer->hidden;
     gu.I = layer->intermediate;
@@ -201,8 +211,8 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     dn.hidden = w.hidden;
     dn.experts = layer->d_experts;
     dn.seg = gu.seg;
-    dn.out_row = w.draw_indices;
-    dn.weight = w.weights_by_position;
+    dn.out_row = slots_direct ? nullptr : w.draw_indices;
+    dn.weight = slots_direct ? d_topk_weights : w.weights_by_position;
     dn.contrib = w.contrib;
     dn.H = layer->hidden;
     dn.I = layer->intermediate;

@@ -258,11 +258,12 @@ def test_layer_on_minimal_shapes(orc, H, I, B):
     assert np.abs(out - want).max() <= 6e-3 * np.abs(want).max()
 
 
-@pytest.mark.parametrize("T", [6, 150])
+@pytest.mark.parametrize("T", [1, 6, 150])
 def test_out_of_range_ids_contribute_nothing(orc, T):
     """An id outside [0, experts) is dropped by the permutation (as the reference's does); the
     slot-ordered reduce must then leave that slot out instead of adding a row nobody wrote. Run
-    on the decode (segment) path and on the grouped path, after a call that left other values in
+    on the single-token path (which reads the ids directly; all three of its slots are bad), on
+    the decode (segment) path and on the grouped path, after a call that left other values in
     the workspace."""
     torch, h, capi, moe, synth = _setup()
     H, I, E, k, limit = 256, 256, 12, 3, 7.0
@@ -276,11 +277,11 @@ def test_out_of_range_ids_contribute_nothing(orc, T):
     d_x = h.dev_half(x)
     layer.routed(d_x, h.to_dev(ids), h.to_dev(w))          # fills every contribution row
     bad = ids.copy()
-    bad[1, 0], bad[T - 1, k - 1], bad[2, 1] = -1, E, 1 << 20
+    bad[min(1, T - 1), 0], bad[T - 1, k - 1], bad[min(2, T - 1), 1] = -1, E, 1 << 20
     out = layer.routed(d_x, h.to_dev(bad), h.to_dev(w)).cpu().numpy()
     experts = {e: h.Expert(31, e, H, I) for e in range(E)}
     shared = h.Expert(31, E, H, I)
-    check = [0, 1, 2, T - 1]
+    check = sorted({0, min(1, T - 1), min(2, T - 1), T - 1})
     want = np.zeros((len(check), H))
     for n, t in enumerate(check):
         keep = [s for s in range(k) if 0 <= bad[t, s] < E]
@@ -288,6 +289,33 @@ def test_out_of_range_ids_contribute_nothing(orc, T):
         want[n] = row[0]
     assert np.isfinite(out).all()
     assert np.abs(out[check] - want).max() <= 6e-3 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("shared", [True, False])
+def test_single_token_reads_its_slots_directly(orc, shared):
+    """One token takes no permutation launch: the kernels read its ids and weights as they are.
+    Its result has to be the one the same token gets as row 0 of a two-token batch (which goes
+    through the permutation), bit for bit -- same kernels, same summation order -- and the
+    oracle's; without an always-on expert the routed sum is added to what the output holds."""
+    torch, h, capi, moe, synth = _setup()
+    H, I, E, k, limit = 512, 384, 10, 4, 7.0
+    pool = moe.ExpertPool(E + (1 if shared else 0), H, I)
+    assert pool.fill_synthetic(seed=33, first_expert_id=0) == 0
+    layer = moe.MoeLayer(pool, E, k, shared, limit)
+    ids = np.array([[7, 2, 9, 0], [1, 2, 3, 4]], dtype=np.int32)
+    w = synth.route_weights(33, 2 * k).reshape(2, k).astype(np.float32)
+    x = synth.activations(33, 2, H)
+    d_x, d_ids, d_w = h.dev_half(x), h.to_dev(ids), h.to_dev(w)
+    start = synth.activations(34, 2, H).astype(np.float16)
+    pair = layer.routed(d_x, d_ids, d_w, out=h.to_dev(start.copy())).cpu().numpy()
+    one = layer.routed(d_x[:1], d_ids[:1], d_w[:1], out=h.to_dev(start[:1].copy())).cpu().numpy()
+    assert np.array_equal(one[0], pair[0])
+    experts = {int(e): h.Expert(33, int(e), H, I) for e in ids[0]}
+    sh = h.Expert(33, E, H, I) if shared else None
+    want = _oracle_layer(orc, h, experts, x[:1], ids[:1], w[:1], sh, limit)[0]
+    if not shared:
+        want = want + start[0].astype(np.float64)
+    assert np.abs(one[0] - want).max() <= 6e-3 * np.abs(want).max()
 
 
 def test_decode_segments_of_two_token_tiles(orc):
