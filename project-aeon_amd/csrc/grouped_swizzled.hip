@@ -3,11 +3,11 @@
 // through the 8-slot by-value tables). They read the payload in place, so they stay valid when
 // the caller recycles its expert slots; the resident fast path is the wave64-packed one.
 //
-// One workgroup = (expert, 16-position token tile, four 16-row weight tiles, one per wave).
-// For each 32-column group, lane (row l%16, chunk l/16) fetches word `chunk` of the row's
-// storage slot and the slot's fp16 scale, dequantises to fp16 with one rounding per weight
-// (the feed rule of the reference's grouped path, __hmul2(unpack2, scale)), and issues one
-// v_mfma_f32_16x16x32_f16 against the token tile's activations.
+// One workgroup = (expert, window of up to 64 positions, four 16-row weight tiles, one per wave).
+// Per 128 columns, lane (row l%16, chunk l/16) fetches the row's 16-byte storage slot of
+// 32-group 4G+chunk and its fp16 scale, dequantises to fp16 with one rounding per weight (the
+// feed rule of the reference's grouped path, __hmul2(unpack2, scale)), and issues four
+// v_mfma_f32_16x16x32_f16 per token tile against the activations of the same columns.
 #include "common.hpp"
 
 namespace aeon355 {
@@ -29,15 +29,14 @@ struct GroupedSwzArgs {
     float limit;
 };
 
-template <int RPW, int LPR, bool GATE_UP>
-__global__ __launch_bounds__(256) void grouped_swizzled_kernel(GroupedSwzArgs a) {
-    const int expert = blockIdx.y;
-    if (expert >= a.expert_count) return;
-    const int first = a.expert_offsets[expert];
-    const int count = a.expert_offsets[expert + 1] - first;
-    const int m0 = blockIdx.z * 16;
-    if (m0 >= count) return;
+constexpr int kSwzWindowTiles = 4;  // token tiles of 16 positions one workgroup carries
 
+// MT token tiles ride on one pass over the weights: a fragment is fetched and dequantised once
+// and multiplied into each tile. A token's own sum over K keeps its order whatever MT is, so
+// the result does not depend on how an expert's positions fall into windows.
+template <int RPW, int LPR, bool GATE_UP, int MT>
+__device__ __forceinline__ void grouped_swizzled_window(const GroupedSwzArgs& a, int expert, int first,
+                                                        int count, int m0) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int n = lane & 15;
@@ -53,66 +52,124 @@ __global__ __launch_bounds__(256) void grouped_swizzled_kernel(GroupedSwzArgs a)
     const uint32_t* pb = GATE_UP ? static_cast<const uint32_t*>(a.w13.w3[expert]) : nullptr;
     const uint16_t* sb = GATE_UP ? static_cast<const uint16_t*>(a.w13.s3[expert]) : nullptr;
 
-    // a padded token column repeats the tile's last live position; its results are not stored
-    const int m = m0 + n < count ? m0 + n : count - 1;
-    const uint16_t* xrow;
-    if (GATE_UP) {
-        xrow = a.activation + static_cast<size_t>(a.token_indices[first + m]) * a.activation_stride;
-    } else {
-        xrow = a.activation + (static_cast<size_t>(expert) * a.hidden_tokens + m) * a.K;
+    // a padded token column repeats the window's last live position; its results are not stored
+    const uint16_t* xrow[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = m0 + mt * 16 + n < count ? m0 + mt * 16 + n : count - 1;
+        if (GATE_UP) {
+            xrow[mt] = a.activation + static_cast<size_t>(a.token_indices[first + m]) * a.activation_stride;
+        } else {
+            xrow[mt] = a.activation + (static_cast<size_t>(expert) * a.hidden_tokens + m) * a.K;
+        }
     }
-    xrow += chunk * 8;
 
     const size_t slot_base = (static_cast<size_t>(row / RPW) * iterations) * 32 + (row % RPW) * LPR;
-    float4_t acc_a = {0.0f, 0.0f, 0.0f, 0.0f};
-    float4_t acc_b = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (int g = 0; g < groups32; ++g) {
+    float4_t acc_a[MT], acc_b[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        acc_a[mt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        acc_b[mt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    // The matrix instruction sums over k whatever order the lanes agree on, so per 128 columns
+    // lane (row, chunk) takes the whole 16-byte slot of 32-group 4G+chunk (one load, one scale)
+    // and in step j multiplies its word j with the activations of the same eight columns:
+    // four steps cover the lane's slot, the four chunks cover the 128 columns.
+    auto dequant = [&](uint32_t word, half_t scale) {
+        half2_t p[4];
+        unpack8(word, p);
+        const half2_t s2 = {scale, scale};
+        const half8_t w = {(p[0] * s2)[0], (p[0] * s2)[1], (p[1] * s2)[0], (p[1] * s2)[1],
+                           (p[2] * s2)[0], (p[2] * s2)[1], (p[3] * s2)[0], (p[3] * s2)[1]};
+        return w;
+    };
+    const uint4* qa = reinterpret_cast<const uint4*>(pa);
+    const uint4* qb = reinterpret_cast<const uint4*>(pb);
+    for (int G = 0; G < groups32 / 4; ++G) {
+        const int g = 4 * G + chunk;
         const size_t slot = slot_base + static_cast<size_t>(g / LPR) * 32 + g % LPR;
-        const half8_t x = *reinterpret_cast<const half8_t*>(xrow + g * 32);
-        {
-            union { uint16_t u; half_t h; } s;
-            s.u = sa[slot];
-            half2_t p[4];
-            unpack8(pa[slot * 4 + chunk], p);
-            const half2_t s2 = {s.h, s.h};
-            const half8_t w = {(p[0] * s2)[0], (p[0] * s2)[1], (p[1] * s2)[0], (p[1] * s2)[1],
-                               (p[2] * s2)[0], (p[2] * s2)[1], (p[3] * s2)[0], (p[3] * s2)[1]};
-            acc_a = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, x, acc_a, 0, 0, 0);
-        }
+        const uint4 wa4 = qa[slot];
+        union { uint16_t u; half_t h; } s_a, s_b;
+        s_a.u = sa[slot];
+        uint4 wb4 = make_uint4(0, 0, 0, 0);
+        s_b.u = 0;
         if (GATE_UP) {
-            union { uint16_t u; half_t h; } s;
-            s.u = sb[slot];
-            half2_t p[4];
-            unpack8(pb[slot * 4 + chunk], p);
-            const half2_t s2 = {s.h, s.h};
-            const half8_t w = {(p[0] * s2)[0], (p[0] * s2)[1], (p[1] * s2)[0], (p[1] * s2)[1],
-                               (p[2] * s2)[0], (p[2] * s2)[1], (p[3] * s2)[0], (p[3] * s2)[1]};
-            acc_b = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, x, acc_b, 0, 0, 0);
+            wb4 = qb[slot];
+            s_b.u = sb[slot];
+        }
+        half8_t x[MT][4];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                x[mt][j] = *reinterpret_cast<const half8_t*>(xrow[mt] + g * 32 + j * 8);
+            }
+        const uint32_t wa[4] = {wa4.x, wa4.y, wa4.z, wa4.w};
+        const uint32_t wb[4] = {wb4.x, wb4.y, wb4.z, wb4.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const half8_t fa = dequant(wa[j], s_a.h);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                acc_a[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa, x[mt][j], acc_a[mt], 0, 0, 0);
+            }
+            if (GATE_UP) {
+                const half8_t fb = dequant(wb[j], s_b.h);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    acc_b[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb, x[mt][j], acc_b[mt], 0, 0, 0);
+                }
+            }
         }
     }
 
-    if (m0 + n >= count) return;
     const int row0 = tile * 16 + chunk * 4;  // this lane holds output rows row0..row0+3 of token n
-    if (GATE_UP) {
-        uint16_t* out = a.expert_hidden +
-                        (static_cast<size_t>(expert) * a.hidden_tokens + m0 + n) * a.N + row0;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            out[i] = float_to_half_bits(clamped_swiglu(acc_a[i], acc_b[i], a.limit));
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = m0 + mt * 16 + n;
+        if (m >= count) continue;
+        if (GATE_UP) {
+            uint16_t* out = a.expert_hidden +
+                            (static_cast<size_t>(expert) * a.hidden_tokens + m) * a.N + row0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                out[i] = float_to_half_bits(clamped_swiglu(acc_a[mt][i], acc_b[mt][i], a.limit));
+            }
+        } else {
+            const int position = first + m;
+            const float w = a.draw_weights[position];
+            float* out = a.contrib + static_cast<size_t>(a.draw_indices[position]) * a.N + row0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out[i] = w * acc_a[mt][i];
         }
+    }
+}
+
+template <int RPW, int LPR, bool GATE_UP>
+__global__ __launch_bounds__(256) void grouped_swizzled_kernel(GroupedSwzArgs a) {
+    const int expert = blockIdx.y;
+    if (expert >= a.expert_count) return;
+    const int first = a.expert_offsets[expert];
+    const int count = a.expert_offsets[expert + 1] - first;
+    const int m0 = blockIdx.z * (kSwzWindowTiles * 16);
+    if (m0 >= count) return;
+    const int live = (count - m0 + 15) / 16;
+    if (live >= 4) {
+        grouped_swizzled_window<RPW, LPR, GATE_UP, 4>(a, expert, first, count, m0);
+    } else if (live == 3) {
+        grouped_swizzled_window<RPW, LPR, GATE_UP, 3>(a, expert, first, count, m0);
+    } else if (live == 2) {
+        grouped_swizzled_window<RPW, LPR, GATE_UP, 2>(a, expert, first, count, m0);
     } else {
-        const int position = first + m0 + n;
-        const float w = a.draw_weights[position];
-        float* out = a.contrib + static_cast<size_t>(a.draw_indices[position]) * a.N + row0;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) out[i] = w * acc_a[i];
+        grouped_swizzled_window<RPW, LPR, GATE_UP, 1>(a, expert, first, count, m0);
     }
 }
 
 template <bool GATE_UP>
 static int launch_grouped_swizzled(const GroupedSwzArgs& a, int rpw, int lpr, hipStream_t stream,
                                    const char* who) {
-    const dim3 grid((a.N / 16 + 3) / 4, a.expert_count, (a.hidden_tokens + 15) / 16);
+    const dim3 grid((a.N / 16 + 3) / 4, a.expert_count,
+                    (a.hidden_tokens + kSwzWindowTiles * 16 - 1) / (kSwzWindowTiles * 16));
     if (rpw == 4 && lpr == 8) {
         grouped_swizzled_kernel<4, 8, GATE_UP><<<grid, 256, 0, stream>>>(a);
     } else if (rpw == 8 && lpr == 4) {
@@ -142,7 +199,7 @@ extern "C" int aeon_moe_grouped_w13_swiglu(const void* d_activation, const int* 
                  AEON_ERR_INVALID_ARGUMENT, "%s: expert count out of range", who);
     if (activation_stride == 0) activation_stride = K;
     AEON_REQUIRE(rpw > 0 && lpr > 0 && rpw * lpr == 32 && N > 0 && N % 16 == 0 && N % rpw == 0 &&
-                     K > 0 && K % 64 == 0 && (K / 32) % lpr == 0 && activation_stride >= K &&
+                     K > 0 && K % 128 == 0 && (K / 32) % lpr == 0 && activation_stride >= K &&
                      activation_stride % 8 == 0 && expert_hidden_tokens > 0,
                  AEON_ERR_INVALID_ARGUMENT, "%s: incompatible N/K shape", who);
     GroupedSwzArgs a{};
@@ -172,7 +229,7 @@ extern "C" int aeon_moe_grouped_w2(const void* d_expert_hidden, const int* d_exp
     AEON_REQUIRE(expert_count > 0 && expert_count <= AEON_SWIZZLED_MAX_EXPERTS,
                  AEON_ERR_INVALID_ARGUMENT, "%s: expert count out of range", who);
     AEON_REQUIRE(rpw > 0 && lpr > 0 && rpw * lpr == 32 && N > 0 && N % 16 == 0 && N % rpw == 0 &&
-                     K > 0 && K % 64 == 0 && (K / 32) % lpr == 0 && expert_hidden_tokens > 0,
+                     K > 0 && K % 128 == 0 && (K / 32) % lpr == 0 && expert_hidden_tokens > 0,
                  AEON_ERR_INVALID_ARGUMENT, "%s: incompatible N/K shape", who);
     GroupedSwzArgs a{};
     a.activation = static_cast<const uint16_t*>(d_expert_hidden);
