@@ -103,6 +103,108 @@ def calibrate_mfma(capi, torch):
     return out
 
 
+def run_dropin(capi, moe, torch, np):
+    """The entry points that read the reference's `.aeon` layout in place, at the reference's own
+    shape (hidden 4096, intermediate 2048, top-6, one scale per 32 columns, 13.5 MiB per expert):
+    the per-token trio (gate/up, W2 contribution, fixed-order reduce) and a chunk through the
+    permutation and the grouped launches in windows of eight experts, as
+    run_moe_grouped_expert_batch issues them. 64 resident experts, random payload bytes."""
+    H, I, K, NE, limit = 4096, 2048, 6, 64, 10.0
+    sp = moe.stream_ptr
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1)
+
+    def words(n):
+        return torch.randint(-2**31, 2**31 - 1, (n,), dtype=torch.int32, device="cuda", generator=gen)
+
+    def scales(n):
+        e = torch.randint(0, 4, (n,), device="cuda", generator=gen)
+        return torch.ldexp(torch.ones(n, device="cuda"), (e - 7).float()).half()
+
+    experts = [{name: (words(r * c // 8), scales(r * c // 32))
+                for name, r, c in (("w1", I, H), ("w3", I, H), ("w2", H, I))} for _ in range(NE)]
+    expert_bytes = 3 * (I * H // 2 + I * H // 32 * 2)
+
+    def tables(ids):
+        w13, w2 = capi.W13Table(), capi.W2Table()
+        for j, e in enumerate(ids):
+            m = experts[e]
+            w13.w1[j], w13.s1[j] = m["w1"][0].data_ptr(), m["w1"][1].data_ptr()
+            w13.w3[j], w13.s3[j] = m["w3"][0].data_ptr(), m["w3"][1].data_ptr()
+            w2.w2[j], w2.s2[j] = m["w2"][0].data_ptr(), m["w2"][1].data_ptr()
+        return w13, w2
+
+    res = {"shape": {"hidden": H, "intermediate": I, "top_k": K, "experts": NE, "scale_group": 32}}
+    x = (torch.rand(H, device="cuda") - 0.5).half()
+    hidden = torch.zeros(8, I, dtype=torch.float16, device="cuda")
+    contrib = torch.zeros(K, H, dtype=torch.float32, device="cuda")
+    out = torch.zeros(H, dtype=torch.float16, device="cuda")
+    wts = torch.full((K,), 1.0 / K, device="cuda")
+    tabs = [tables([(K * t + j) % NE for j in range(K)]) for t in range(32)]
+
+    def token(i):
+        w13, w2 = tabs[i % len(tabs)]
+        capi.call("aeon_moe_gemv_w13_swiglu", capi.vp(x), C.byref(w13), capi.vp(hidden), None, I, K, I,
+                  H, 4, 8, C.c_float(limit), sp())
+        capi.call("aeon_moe_fused_w2_contrib", capi.vp(hidden), C.byref(w2), capi.vp(wts),
+                  capi.vp(contrib), K, H, I, 8, 4, sp())
+        capi.call("aeon_moe_accumulate_fixed_order", capi.vp(contrib), K, capi.vp(out), capi.vp(out),
+                  H, sp())
+
+    settle(token, torch)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for i in range(320):
+        token(i)
+    b.record()
+    torch.cuda.synchronize()
+    ms = a.elapsed_time(b) / 320
+    res["token_trio"] = {"ms_per_token": round(ms, 4),
+                         "weights_gbps": round(K * expert_bytes / ms / 1e6, 1)}
+    res["chunks"] = []
+    for T in (64, 256, 1024):
+        rng = np.random.default_rng(T)
+        ids_h = np.stack([rng.permutation(NE)[:K] for _ in range(T)]).astype(np.int32)
+        ids = torch.from_numpy(ids_h).cuda()
+        w = torch.full((T, K), 1.0 / K, device="cuda")
+        xin = (torch.rand(T, H, device="cuda") - 0.5).half()
+        draws = T * K
+        off = torch.zeros(NE + 1, dtype=torch.int32, device="cuda")
+        tok = torch.zeros(draws, dtype=torch.int32, device="cuda")
+        drw = torch.zeros_like(tok)
+        wp = torch.zeros(draws, device="cuda")
+        widest = int(np.bincount(ids_h.ravel(), minlength=NE).max())
+        chunk_hidden = torch.zeros(8 * widest * I, dtype=torch.float16, device="cuda")
+        cont = torch.zeros(draws, H, dtype=torch.float32, device="cuda")
+        outb = torch.zeros(T, H, dtype=torch.float16, device="cuda")
+        wins = [tables(list(range(w0, w0 + 8))) for w0 in range(0, NE, 8)]
+
+        def chunk(i):
+            capi.call("aeon_expert_permutation", capi.vp(ids), T, K, NE, capi.vp(off), capi.vp(tok),
+                      capi.vp(drw), capi.vp(w), capi.vp(wp), sp())
+            for n, (w13, w2) in enumerate(wins):
+                bounds = C.c_void_p(off.data_ptr() + 4 * 8 * n)
+                capi.call("aeon_moe_grouped_w13_swiglu", capi.vp(xin), bounds, capi.vp(tok),
+                          C.byref(w13), capi.vp(chunk_hidden), 8, widest, I, H, 4, 8,
+                          C.c_float(limit), H, sp())
+                capi.call("aeon_moe_grouped_w2", capi.vp(chunk_hidden), bounds, capi.vp(drw),
+                          capi.vp(wp), C.byref(w2), capi.vp(cont), 8, widest, H, I, 8, 4, sp())
+            capi.call("aeon_moe_accumulate_fixed_order_tokens", capi.vp(cont), T, K, capi.vp(outb), H,
+                      H, sp())
+
+        settle(chunk, torch)
+        a.record()
+        for i in range(20):
+            chunk(i)
+        b.record()
+        torch.cuda.synchronize()
+        ms = a.elapsed_time(b) / 20
+        res["chunks"].append({"tokens": T, "tokens_per_expert": round(draws / NE, 1),
+                              "ms": round(ms, 3),
+                              "tflops": round(2.0 * draws * 3 * H * I / ms / 1e9, 1)})
+    return res
+
+
 def run_prefill(layer, moe, capi, synth, torch, np, H, I, E, K_TOP, SEED, steps, warmup):
     """BASELINE config 3: 2048 tokens, top-8 of 256 experts with Zipf(1.1) popularity, through the
     permutation -> grouped gate+up GEMM + SwiGLU -> grouped W2 GEMM -> fixed-order reduce path.
@@ -306,6 +408,9 @@ def main():
     ap.add_argument("--calibrate-mfma", action="store_true",
                     help="only measure the sustained fp16 MFMA rate (register-resident loop with "
                          "constant and with random operands) and a library fp16 GEMM, for context")
+    ap.add_argument("--dropin", action="store_true",
+                    help="only time the entry points that read the .aeon layout in place, at the "
+                         "reference's own shape (hidden 4096, top-6, one scale per 32 columns)")
     ap.add_argument("--sweep", action="store_true",
                     help="also report batch 1/8/32/64 in the `sweep` field")
     args = ap.parse_args()
@@ -344,6 +449,9 @@ def main():
         return
     if args.calibrate_mfma:
         print(json.dumps(calibrate_mfma(capi, torch)))
+        return
+    if args.dropin:
+        print(json.dumps({"dropin": run_dropin(capi, moe, torch, np)}))
         return
     H, I, E, K_TOP, LIMIT, SEED = 7168, 2048, args.experts, 8, 7.0, 0
     B = args.batch

@@ -34,22 +34,35 @@ constexpr int kSwzWindowTiles = 4;  // token tiles of 16 positions one workgroup
 // MT token tiles ride on one pass over the weights: a fragment is fetched and dequantised once
 // and multiplied into each tile. A token's own sum over K keeps its order whatever MT is, so
 // the result does not depend on how an expert's positions fall into windows.
+//
+// The matrix instruction sums over k whatever order the lanes agree on, so per 128 columns lane
+// (row, chunk) takes the whole 16-byte slot of 32-group 4G+chunk (one load, one scale) and in
+// step j multiplies its word j with the activations of the same eight columns: four steps
+// cover the lane's slot, the four chunks cover the 128 columns.
+//
+// The four waves of a workgroup hold different weight rows and the same activations, so each
+// wave fetches one step's activation fragments (j = its index) a group ahead and all four read
+// them from LDS: one barrier per 128 columns, two LDS buffers (the one written in pass G was
+// last read in pass G-1, before that pass's barrier). Weights and scales are fetched one pass
+// ahead into registers.
 template <int RPW, int LPR, bool GATE_UP, int MT>
 __device__ __forceinline__ void grouped_swizzled_window(const GroupedSwzArgs& a, int expert, int first,
-                                                        int count, int m0) {
+                                                        int count, int m0, half8_t* xs) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int n = lane & 15;
     const int chunk = lane >> 4;
-    const int tile = blockIdx.x * 4 + wave;
-    if (tile * 16 >= a.N) return;
+    const int tile_here = blockIdx.x * 4 + wave;
+    const bool live_wave = tile_here * 16 < a.N;   // a wave past the last row tile still serves
+    const int tile = live_wave ? tile_here : 0;    // the barriers and the activation fetch
     const int row = tile * 16 + n;  // the A operand's row
     const int groups32 = a.K / 32;
     const int iterations = groups32 / LPR;
+    const int passes = groups32 / 4;
 
-    const uint32_t* pa = static_cast<const uint32_t*>(GATE_UP ? a.w13.w1[expert] : a.w2.w2[expert]);
+    const uint4* qa = static_cast<const uint4*>(GATE_UP ? a.w13.w1[expert] : a.w2.w2[expert]);
     const uint16_t* sa = static_cast<const uint16_t*>(GATE_UP ? a.w13.s1[expert] : a.w2.s2[expert]);
-    const uint32_t* pb = GATE_UP ? static_cast<const uint32_t*>(a.w13.w3[expert]) : nullptr;
+    const uint4* qb = GATE_UP ? static_cast<const uint4*>(a.w13.w3[expert]) : nullptr;
     const uint16_t* sb = GATE_UP ? static_cast<const uint16_t*>(a.w13.s3[expert]) : nullptr;
 
     // a padded token column repeats the window's last live position; its results are not stored
@@ -62,67 +75,95 @@ __device__ __forceinline__ void grouped_swizzled_window(const GroupedSwzArgs& a,
         } else {
             xrow[mt] = a.activation + (static_cast<size_t>(expert) * a.hidden_tokens + m) * a.K;
         }
+        xrow[mt] += chunk * 32 + wave * 8;   // this wave's step of this lane's slot
     }
+    auto x_fragment = [&](int mt, int G) {
+        return *reinterpret_cast<const half8_t*>(xrow[mt] + G * 128);
+    };
+    auto lds = [&](int buffer, int mt, int j) { return xs + ((buffer * kSwzWindowTiles + mt) * 4 + j) * 64 + lane; };
 
     const size_t slot_base = (static_cast<size_t>(row / RPW) * iterations) * 32 + (row % RPW) * LPR;
+    auto slot_of = [&](int G) {
+        const int g = 4 * G + chunk;
+        return slot_base + static_cast<size_t>(g / LPR) * 32 + g % LPR;
+    };
     float4_t acc_a[MT], acc_b[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         acc_a[mt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
         acc_b[mt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
     }
-    // The matrix instruction sums over k whatever order the lanes agree on, so per 128 columns
-    // lane (row, chunk) takes the whole 16-byte slot of 32-group 4G+chunk (one load, one scale)
-    // and in step j multiplies its word j with the activations of the same eight columns:
-    // four steps cover the lane's slot, the four chunks cover the 128 columns.
-    auto dequant = [&](uint32_t word, half_t scale) {
+    auto dequant = [&](uint32_t word, uint16_t scale_bits) {
+        union { uint16_t u; half_t h; } s;
+        s.u = scale_bits;
         half2_t p[4];
         unpack8(word, p);
-        const half2_t s2 = {scale, scale};
+        const half2_t s2 = {s.h, s.h};
         const half8_t w = {(p[0] * s2)[0], (p[0] * s2)[1], (p[1] * s2)[0], (p[1] * s2)[1],
                            (p[2] * s2)[0], (p[2] * s2)[1], (p[3] * s2)[0], (p[3] * s2)[1]};
         return w;
     };
-    const uint4* qa = reinterpret_cast<const uint4*>(pa);
-    const uint4* qb = reinterpret_cast<const uint4*>(pb);
-    for (int G = 0; G < groups32 / 4; ++G) {
-        const int g = 4 * G + chunk;
-        const size_t slot = slot_base + static_cast<size_t>(g / LPR) * 32 + g % LPR;
-        const uint4 wa4 = qa[slot];
-        union { uint16_t u; half_t h; } s_a, s_b;
-        s_a.u = sa[slot];
-        uint4 wb4 = make_uint4(0, 0, 0, 0);
-        s_b.u = 0;
+
+    uint4 wa4 = qa[slot_of(0)];
+    uint16_t s_a = sa[slot_of(0)];
+    uint4 wb4 = make_uint4(0, 0, 0, 0);
+    uint16_t s_b = 0;
+    if (GATE_UP) {
+        wb4 = qb[slot_of(0)];
+        s_b = sb[slot_of(0)];
+    }
+    half8_t xr[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) *lds(0, mt, wave) = x_fragment(mt, 0);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) xr[mt] = x_fragment(mt, passes > 1 ? 1 : 0);
+    __syncthreads();
+
+    for (int G = 0; G < passes; ++G) {
+        const int next = G + 1 < passes ? G + 1 : G;
+        const uint4 wa4n = qa[slot_of(next)];
+        const uint16_t s_an = sa[slot_of(next)];
+        uint4 wb4n = make_uint4(0, 0, 0, 0);
+        uint16_t s_bn = 0;
         if (GATE_UP) {
-            wb4 = qb[slot];
-            s_b.u = sb[slot];
+            wb4n = qb[slot_of(next)];
+            s_bn = sb[slot_of(next)];
         }
         half8_t x[MT][4];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                x[mt][j] = *reinterpret_cast<const half8_t*>(xrow[mt] + g * 32 + j * 8);
-            }
+            for (int j = 0; j < 4; ++j) x[mt][j] = *lds(G & 1, mt, j);
         const uint32_t wa[4] = {wa4.x, wa4.y, wa4.z, wa4.w};
         const uint32_t wb[4] = {wb4.x, wb4.y, wb4.z, wb4.w};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const half8_t fa = dequant(wa[j], s_a.h);
+            const half8_t fa = dequant(wa[j], s_a);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 acc_a[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa, x[mt][j], acc_a[mt], 0, 0, 0);
             }
             if (GATE_UP) {
-                const half8_t fb = dequant(wb[j], s_b.h);
+                const half8_t fb = dequant(wb[j], s_b);
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
                     acc_b[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb, x[mt][j], acc_b[mt], 0, 0, 0);
                 }
             }
         }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) *lds((G + 1) & 1, mt, wave) = xr[mt];
+        const int after = G + 2 < passes ? G + 2 : passes - 1;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) xr[mt] = x_fragment(mt, after);
+        wa4 = wa4n;
+        s_a = s_an;
+        wb4 = wb4n;
+        s_b = s_bn;
+        __syncthreads();
     }
 
+    if (!live_wave) return;
     const int row0 = tile * 16 + chunk * 4;  // this lane holds output rows row0..row0+3 of token n
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -147,6 +188,7 @@ __device__ __forceinline__ void grouped_swizzled_window(const GroupedSwzArgs& a,
 
 template <int RPW, int LPR, bool GATE_UP>
 __global__ __launch_bounds__(256) void grouped_swizzled_kernel(GroupedSwzArgs a) {
+    __shared__ half8_t xs[2 * kSwzWindowTiles * 4 * 64];
     const int expert = blockIdx.y;
     if (expert >= a.expert_count) return;
     const int first = a.expert_offsets[expert];
@@ -155,13 +197,13 @@ __global__ __launch_bounds__(256) void grouped_swizzled_kernel(GroupedSwzArgs a)
     if (m0 >= count) return;
     const int live = (count - m0 + 15) / 16;
     if (live >= 4) {
-        grouped_swizzled_window<RPW, LPR, GATE_UP, 4>(a, expert, first, count, m0);
+        grouped_swizzled_window<RPW, LPR, GATE_UP, 4>(a, expert, first, count, m0, xs);
     } else if (live == 3) {
-        grouped_swizzled_window<RPW, LPR, GATE_UP, 3>(a, expert, first, count, m0);
+        grouped_swizzled_window<RPW, LPR, GATE_UP, 3>(a, expert, first, count, m0, xs);
     } else if (live == 2) {
-        grouped_swizzled_window<RPW, LPR, GATE_UP, 2>(a, expert, first, count, m0);
+        grouped_swizzled_window<RPW, LPR, GATE_UP, 2>(a, expert, first, count, m0, xs);
     } else {
-        grouped_swizzled_window<RPW, LPR, GATE_UP, 1>(a, expert, first, count, m0);
+        grouped_swizzled_window<RPW, LPR, GATE_UP, 1>(a, expert, first, count, m0, xs);
     }
 }
 
