@@ -43,8 +43,8 @@ constexpr int kSwzWindowTiles = 4;  // token tiles of 16 positions one workgroup
 // The four waves of a workgroup hold different weight rows and the same activations, so each
 // wave fetches one step's activation fragments (j = its index) a group ahead and all four read
 // them from LDS: one barrier per 128 columns, two LDS buffers (the one written in pass G was
-// last read in pass G-1, before that pass's barrier). Weights and scales are fetched one pass
-// ahead into registers.
+// last read in pass G-1, before that pass's barrier). Weights and scales wait in a register
+// ring three passes deep.
 template <int RPW, int LPR, bool GATE_UP, int MT>
 __device__ __forceinline__ void grouped_swizzled_window(const GroupedSwzArgs& a, int expert, int first,
                                                         int count, int m0, half8_t* xs) {
@@ -104,47 +104,55 @@ __device__ __forceinline__ void grouped_swizzled_window(const GroupedSwzArgs& a,
         return w;
     };
 
-    uint4 wa4 = qa[slot_of(0)];
-    uint16_t s_a = sa[slot_of(0)];
-    uint4 wb4 = make_uint4(0, 0, 0, 0);
-    uint16_t s_b = 0;
-    if (GATE_UP) {
-        wb4 = qb[slot_of(0)];
-        s_b = sb[slot_of(0)];
-    }
+    // Ring of kDepth passes of weights and scales in registers. Requests are kept in one order
+    // everywhere (the next activation fragments, then the weights kDepth passes ahead): the
+    // compiler's wait counts are static, so the order before the loop has to be the loop's.
+    constexpr int kDepth = 3;
+    uint4 wa4[kDepth], wb4[kDepth];
+    uint16_t s_a[kDepth], s_b[kDepth];
+    auto fetch_weights = [&](int d, int G) {
+        const size_t slot = slot_of(G < passes ? G : passes - 1);
+        wa4[d] = qa[slot];
+        s_a[d] = sa[slot];
+        if (GATE_UP) {
+            wb4[d] = qb[slot];
+            s_b[d] = sb[slot];
+        } else {
+            wb4[d] = make_uint4(0, 0, 0, 0);
+            s_b[d] = 0;
+        }
+    };
     half8_t xr[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) *lds(0, mt, wave) = x_fragment(mt, 0);
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) xr[mt] = x_fragment(mt, passes > 1 ? 1 : 0);
+    for (int d = 0; d < kDepth; ++d) {
+        if (d == kDepth - 1) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) xr[mt] = x_fragment(mt, passes > 1 ? 1 : 0);
+        }
+        fetch_weights(d, d);
+        __builtin_amdgcn_sched_barrier(0);
+    }
     __syncthreads();
 
-    for (int G = 0; G < passes; ++G) {
-        const int next = G + 1 < passes ? G + 1 : G;
-        const uint4 wa4n = qa[slot_of(next)];
-        const uint16_t s_an = sa[slot_of(next)];
-        uint4 wb4n = make_uint4(0, 0, 0, 0);
-        uint16_t s_bn = 0;
-        if (GATE_UP) {
-            wb4n = qb[slot_of(next)];
-            s_bn = sb[slot_of(next)];
-        }
+    auto pass = [&](int d, int G) {
         half8_t x[MT][4];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int j = 0; j < 4; ++j) x[mt][j] = *lds(G & 1, mt, j);
-        const uint32_t wa[4] = {wa4.x, wa4.y, wa4.z, wa4.w};
-        const uint32_t wb[4] = {wb4.x, wb4.y, wb4.z, wb4.w};
+        const uint32_t wa[4] = {wa4[d].x, wa4[d].y, wa4[d].z, wa4[d].w};
+        const uint32_t wb[4] = {wb4[d].x, wb4[d].y, wb4[d].z, wb4[d].w};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const half8_t fa = dequant(wa[j], s_a);
+            const half8_t fa = dequant(wa[j], s_a[d]);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 acc_a[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa, x[mt][j], acc_a[mt], 0, 0, 0);
             }
             if (GATE_UP) {
-                const half8_t fb = dequant(wb[j], s_b);
+                const half8_t fb = dequant(wb[j], s_b[d]);
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
                     acc_b[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb, x[mt][j], acc_b[mt], 0, 0, 0);
@@ -156,11 +164,17 @@ __device__ __forceinline__ void grouped_swizzled_window(const GroupedSwzArgs& a,
         const int after = G + 2 < passes ? G + 2 : passes - 1;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) xr[mt] = x_fragment(mt, after);
-        wa4 = wa4n;
-        s_a = s_an;
-        wb4 = wb4n;
-        s_b = s_bn;
+        fetch_weights(d, G + kDepth);   // past the end: the last pass again, unused
         __syncthreads();
+    };
+    int G0 = 0;
+    for (; G0 + kDepth <= passes; G0 += kDepth) {
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d) pass(d, G0 + d);
+    }
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d) {
+        if (G0 + d < passes) pass(d, G0 + d);
     }
 
     if (!live_wave) return;
