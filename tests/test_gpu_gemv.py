@@ -283,3 +283,81 @@ def test_mfma_calibration_loop_runs_and_counts_its_flops():
               None, None)
     torch.cuda.synchronize()
     assert torch.isfinite(sink).all()
+
+
+def test_swizzled_grouped_windows_against_oracle(orc):
+    """The grouped entry points over the `.aeon` layout (distinct group-32 scales) on experts that
+    own 0, 1, 16, 17, 63, 64, 65 and 130 positions: every window size of the kernel, windows that
+    end inside a token tile, an expert split over three windows, an empty expert. Hidden and
+    contributions against the fp64 oracle per position (to 2e-3 of the peak: the feed rounds each
+    scaled weight to fp16); a strided activation buffer gives the
+    same bits as a compact one (tests/test_v4_grouped_wmma_oracle.cpp checks the same)."""
+    torch, h, capi = _setup()
+    from project_aeon_amd import synth
+    H, I, limit = 512, 256, 7.0
+    counts = [0, 1, 16, 17, 63, 64, 65, 130]
+    E, T = len(counts), 140
+    # slot s of token t -> expert: expert e takes its first counts[e] tokens in slot e
+    k = E
+    ids = np.full((T, k), -1, dtype=np.int32)
+    for e, c in enumerate(counts):
+        ids[:c, e] = e
+    weights = synth.route_weights(41, T * k).reshape(T, k).astype(np.float32)
+    x = synth.activations(41, T, H)
+    experts = []
+    rng = np.random.default_rng(41)
+    w13, w2 = capi.W13Table(), capi.W2Table()
+    keep = []
+    for e in range(E):
+        m = {}
+        for name, rows, cols in (("w1", I, H), ("w3", I, H), ("w2", H, I)):
+            packed = rng.integers(0, 2**32, rows * cols // 8, dtype=np.uint64).astype(np.uint32)
+            scale = (0.004 + 0.02 * rng.random(rows * cols // 32)).astype(np.float16).view(np.uint16)
+            m[name] = (packed, scale)
+        experts.append(m)
+        dev = {n: (h.dev_u32(v[0]), h.dev_u16(v[1])) for n, v in m.items()}
+        keep.append(dev)
+        w13.w1[e], w13.s1[e] = dev["w1"][0].data_ptr(), dev["w1"][1].data_ptr()
+        w13.w3[e], w13.s3[e] = dev["w3"][0].data_ptr(), dev["w3"][1].data_ptr()
+        w2.w2[e], w2.s2[e] = dev["w2"][0].data_ptr(), dev["w2"][1].data_ptr()
+    draws = T * k
+    d_ids, d_w = h.to_dev(ids), h.to_dev(weights)
+    off = torch.zeros(E + 1, dtype=torch.int32, device="cuda")
+    tok = torch.zeros(draws, dtype=torch.int32, device="cuda")
+    drw = torch.zeros_like(tok)
+    wp = torch.zeros(draws, device="cuda")
+    capi.call("aeon_expert_permutation", capi.vp(d_ids), T, k, E, capi.vp(off), capi.vp(tok),
+              capi.vp(drw), capi.vp(d_w), capi.vp(wp), h.stream_ptr())
+    widest = max(counts)
+    results = []
+    for stride in (H, H + 64):
+        xin = torch.zeros(T, stride, dtype=torch.float16, device="cuda")
+        xin[:, :H] = h.dev_half(x)
+        hidden = torch.zeros(E * widest * I, dtype=torch.float16, device="cuda")
+        contrib = torch.zeros(draws, H, dtype=torch.float32, device="cuda")
+        capi.call("aeon_moe_grouped_w13_swiglu", capi.vp(xin), capi.vp(off), capi.vp(tok),
+                  C.byref(w13), capi.vp(hidden), E, widest, I, H, 4, 8, C.c_float(limit), stride,
+                  h.stream_ptr())
+        capi.call("aeon_moe_grouped_w2", capi.vp(hidden), capi.vp(off), capi.vp(drw), capi.vp(wp),
+                  C.byref(w2), capi.vp(contrib), E, widest, H, I, 8, 4, h.stream_ptr())
+        torch.cuda.synchronize()
+        results.append((hidden.cpu().numpy().reshape(E, widest, I), contrib.cpu().numpy()))
+    assert np.array_equal(results[0][0], results[1][0]) and np.array_equal(results[0][1], results[1][1])
+    got_hidden, got_contrib = results[0]
+    assert np.array_equal(off.cpu().numpy(), np.concatenate([[0], np.cumsum(counts)]))
+    xf = x.astype(np.float64)
+    for e, c in enumerate(counts):
+        if c == 0:
+            continue
+        m = experts[e]
+        o, hid = orc.expert_ffn(m["w1"], m["w3"], m["w2"], H, I, xf[:c], limit, round_hidden=True,
+                                want_hidden=True)
+        # the grouped feed rounds every weight x scale product to fp16 (the reference's rule,
+        # swizzled_w4a16_feed.hpp:86), so outputs near zero carry errors that are small against
+        # the data's scale and large against themselves: bound |delta| by a fraction of the peak
+        got_h = got_hidden[e, :c].astype(np.float64)
+        assert np.abs(got_h - hid).max() <= 2e-3 * np.abs(hid).max(), (e, c)
+        rows = np.arange(c) * k + e                   # draw index of (token, slot e)
+        want = weights[:c, e].astype(np.float64)[:, None] * o
+        got_c = got_contrib[rows].astype(np.float64)
+        assert np.abs(got_c - want).max() <= 2e-3 * np.abs(want).max(), (e, c)
