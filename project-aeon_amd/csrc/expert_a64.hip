@@ -345,6 +345,23 @@ __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegD
             const float4_t v = {w * acc[0][r][0], w * acc[0][r][1], w * acc[0][r][2], w * acc[0][r][3]};
             const size_t out_row = dn.out_row != nullptr ? dn.out_row[first + n] : first + n;
             *reinterpret_cast<float4_t*>(dn.contrib + out_row * dn.H + row0) = v;
+            if (dn.fused_out != nullptr) {
+                // the reduce over a single slot, with its two roundings kept apart (no fused
+                // multiply-add): the stored fp32 contribution, then one fp16 rounding of the sum
+                const size_t at = static_cast<size_t>(first + n) * dn.H + row0;
+                uint16_t o[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float start = dn.fused_initial != nullptr ? half_bits_to_float(dn.fused_initial[at + i]) : 0.0f;
+                    float product = v[i];
+                    asm volatile("" : "+v"(product));   // keeps the multiply out of an fma with the add
+                    o[i] = float_to_half_bits(start + product);
+                }
+                uint2 packed;
+                packed.x = o[0] | (static_cast<uint32_t>(o[1]) << 16);
+                packed.y = o[2] | (static_cast<uint32_t>(o[3]) << 16);
+                *reinterpret_cast<uint2*>(dn.fused_out + at) = packed;
+            }
         }
     }
 }
@@ -814,7 +831,9 @@ extern "C" int aeon_a64_expert_decode(const void* d_x, int tokens, const aeon_a6
         dn.seg.capacity = 1;
         dn.direct_expert = *expert;
         dn.direct_count = tokens;
-        if (int rc = launch_seg_down(dn, 4, 1, 2, s)) return rc;
+        dn.fused_out = static_cast<uint16_t*>(d_out);
+        dn.fused_initial = static_cast<const uint16_t*>(d_shared);
+        return launch_seg_down(dn, 4, 1, 2, s);   // the reduce over its one slot rides along
     } else {
         GemvArgs g{};
         g.x = static_cast<const uint16_t*>(d_x);

@@ -52,6 +52,11 @@ struct SegDownArgs {
     int H, I;
     aeon_a64_expert direct_expert;
     int direct_count;
+    // Direct mode with a single contribution per token: the K-split kernel also writes
+    // out[token] = half(float(initial[token]) + contribution) (`initial` nullable, may alias
+    // `out`; both [tokens][H]), which is the slot-ordered reduce over one slot.
+    uint16_t* fused_out;
+    const uint16_t* fused_initial;
 };
 
 // k_split: 1, 2 or 4 waves of a workgroup split K between them; 0 = the wide form (four waves,

@@ -259,6 +259,19 @@ def test_config1_one_expert_decode(orc, tokens, use_mfma):
     assert h.rel_err(out.cpu().numpy(), staged) <= TOL
     assert np.abs(out.cpu().numpy() - want).max() <= 6e-3 * np.abs(want).max()
     assert torch.equal(out, contrib.half())
+    # with a starting row (the accumulator the shared expert has already written), also in place:
+    # out = half(float(start) + contrib), fp32 add, one rounding, no fused multiply-add
+    start = h.dev_half(synth.activations(5, tokens, H))
+    out2 = torch.zeros_like(out)
+    capi.call("aeon_a64_expert_decode", capi.vp(d_x), tokens, C.byref(de.c), capi.vp(d_w),
+              capi.vp(hidden), capi.vp(contrib), capi.vp(start), capi.vp(out2), H, I,
+              C.c_float(limit), use_mfma, h.stream_ptr())
+    assert torch.equal(out2, (start.float() + contrib).half())
+    inplace = start.clone()
+    capi.call("aeon_a64_expert_decode", capi.vp(d_x), tokens, C.byref(de.c), capi.vp(d_w),
+              capi.vp(hidden), capi.vp(contrib), capi.vp(inplace), capi.vp(inplace), H, I,
+              C.c_float(limit), use_mfma, h.stream_ptr())
+    assert torch.equal(inplace, out2)
     # against the oracle that keeps hidden in fp64 (dsv4_oracle.hpp:1633-1671) the fp16 store of
     # hidden shows up on near-zero outputs, so that comparison is the reference's own: a fraction
     # of the peak (6e-3, tests/test_v4_expert_oracle.cpp:75-77)
