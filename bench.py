@@ -205,6 +205,34 @@ def run_dropin(capi, moe, torch, np):
     return res
 
 
+def run_chunk_sweep(layer, moe, synth, torch, np, H, I, E, K_TOP, SEED):
+    """The routed step (given ids) at chunk sizes between the decode batch and the 2048-token
+    prefill, uniform and Zipf(1.1) routing: where the step goes from streaming each touched
+    expert once to being bound by the matrix pipe."""
+    be = 3 * matrix_bytes(I, H)
+    rows = []
+    for T in (64, 65, 128, 256, 512, 1024):
+        for s in (0.0, 1.1):
+            ids_h, w_h = synth.zipf_routing(SEED, T, E, K_TOP, s=s)
+            ids = torch.from_numpy(ids_h).cuda()
+            w = torch.from_numpy(w_h).cuda()
+            x = torch.from_numpy(synth.activations(SEED, T, H, unit=3)).cuda()
+            out = torch.empty(T, H, dtype=torch.float16, device="cuda")
+            settle(lambda i: layer.routed(x, ids, w, out), torch, 0.2)
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(20):
+                layer.routed(x, ids, w, out)
+            b.record()
+            torch.cuda.synchronize()
+            ms = a.elapsed_time(b) / 20
+            distinct = int(np.unique(ids_h).size)
+            rows.append({"tokens": T, "zipf_s": s, "distinct_experts": distinct, "ms": round(ms, 3),
+                         "weights_gbps": round((distinct + 1) * be / ms / 1e6, 1),
+                         "tflops": round(2.0 * (T * K_TOP + T) * 3 * H * I / ms / 1e9, 1)})
+    return rows
+
+
 def run_prefill(layer, moe, capi, synth, torch, np, H, I, E, K_TOP, SEED, steps, warmup):
     """BASELINE config 3: 2048 tokens, top-8 of 256 experts with Zipf(1.1) popularity, through the
     permutation -> grouped gate+up GEMM + SwiGLU -> grouped W2 GEMM -> fixed-order reduce path.
@@ -411,6 +439,9 @@ def main():
     ap.add_argument("--dropin", action="store_true",
                     help="only time the entry points that read the .aeon layout in place, at the "
                          "reference's own shape (hidden 4096, top-6, one scale per 32 columns)")
+    ap.add_argument("--chunk-sweep", action="store_true",
+                    help="also time the routed step at 64..1024 tokens (uniform and Zipf routing) "
+                         "into `chunk_sweep`")
     ap.add_argument("--sweep", action="store_true",
                     help="also report batch 1/8/32/64 in the `sweep` field")
     args = ap.parse_args()
@@ -671,6 +702,8 @@ def main():
         result["prefill"] = prefill
     if sweep is not None:
         result["sweep"] = sweep
+    if args.chunk_sweep:
+        result["chunk_sweep"] = run_chunk_sweep(layer, moe, synth, torch, np, H, I, E, K_TOP, SEED)
     print(json.dumps(result))
 
 
