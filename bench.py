@@ -211,7 +211,7 @@ def run_chunk_sweep(layer, moe, synth, torch, np, H, I, E, K_TOP, SEED):
     expert once to being bound by the matrix pipe."""
     be = 3 * matrix_bytes(I, H)
     rows = []
-    for T in (64, 65, 128, 256, 512, 1024):
+    for T in (64, 128, 129, 256, 512, 1024):
         for s in (0.0, 1.1):
             ids_h, w_h = synth.zipf_routing(SEED, T, E, K_TOP, s=s)
             ids = torch.from_numpy(ids_h).cuda()

@@ -14,7 +14,7 @@ extern "C" size_t aeon_router_logits_workspace_bytes(int tokens, int hidden, int
 namespace aeon355 {
 
 // Up to this many tokens a step is a decode batch; above it, a prefill chunk.
-constexpr int kDecodeMaxTokens = 64;
+constexpr int kDecodeMaxTokens = 128;
 
 static size_t align_up(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
 

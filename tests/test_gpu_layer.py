@@ -236,11 +236,13 @@ def test_config2_full_size_sampled(orc):
         assert np.abs(alone[0] - out[t]).max() <= 1e-3 * np.abs(out[t]).max()
 
 
-@pytest.mark.parametrize("H,I,B", [(256, 128, 3), (256, 384, 5), (768, 256, 17), (256, 128, 70)])
+@pytest.mark.parametrize("H,I,B", [(256, 128, 3), (256, 384, 5), (768, 256, 17), (256, 128, 70),
+                                   (256, 128, 128), (256, 128, 129)])
 def test_layer_on_minimal_shapes(orc, H, I, B):
     """Shapes with fewer 128-column groups than a workgroup has K-split waves (a wave with no
     group of its own must not fetch anything outside the matrix), odd group counts for the
-    pipeline tails, and a batch just over the grouped path's threshold on a one-group K."""
+    pipeline tails, and batches at and just over the grouped path's threshold (128 tokens) on a
+    one-group K."""
     torch, h, capi, moe, synth = _setup()
     E, k, limit = 5, 2, 7.0
     pool = moe.ExpertPool(E + 1, H, I)
