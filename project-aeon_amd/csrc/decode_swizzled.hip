@@ -4,15 +4,18 @@
 // The payload stores, per (row block, iteration), 32 uint4 = 512 contiguous bytes: lane
 // row_in_block*LPR + slice holds the 32 columns of group iteration*LPR + slice. A wave64 takes
 // two consecutive iterations at once, so each wave load is 1 KiB contiguous and each scale
-// load 128 B contiguous. A workgroup owns one row block; its waves split K (iterations)
-// between them, every lane keeps all of its loads in flight, and partial sums meet through a
-// wave xor-butterfly and a small LDS exchange. Bandwidth-bound by design: no MFMA.
+// load 128 B contiguous. Each wave of a workgroup owns one row block and walks all of its K in
+// steps of two iterations, up to eight steps of loads in flight per lane; a row's partial sums
+// meet in a wave xor-butterfly, nothing crosses waves. The activations (one row, K halves) are
+// what the four waves share: they are copied into LDS once per workgroup, laid out by 16-byte
+// piece so that neighbouring lanes read neighbouring banks, which takes four of every five
+// vector-memory instructions off the kernel. Bandwidth-bound by design: no MFMA.
 #include "common.hpp"
 
 namespace aeon355 {
 
-constexpr int kWaves = 4;            // waves per workgroup = K splits
-constexpr int kMaxItersPerLane = 8;  // iterations one lane may own (K <= 8*kWaves*2*LPR*32)
+constexpr int kWaves = 4;      // waves per workgroup = row blocks per workgroup
+constexpr int kMaxSteps = 8;   // steps (of two iterations) whose loads one lane keeps in flight
 
 enum class SwzMode { Gemv, Dual, GateUp, W2Contrib, W2Accum };
 
@@ -51,20 +54,25 @@ __global__ __launch_bounds__(kWaves * 64) void swizzled_decode_kernel(SwzArgs a)
     // one writer and a fixed order; every other mode takes its expert from the grid.
     constexpr bool kAccum = MODE == SwzMode::W2Accum;
     constexpr bool kW2 = MODE == SwzMode::W2Contrib || kAccum;
+    extern __shared__ uint4 x_lds[];  // [piece 0..3][32-column group]: the activation row
     const int first_expert = kAccum ? 0 : blockIdx.y;
     const int last_expert = kAccum ? a.expert_count : first_expert + 1;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int half_id = lane >> 5;
     const int lane32 = lane & 31;
-    const int row_block = blockIdx.x;
     const int row_in_block = lane32 / LPR;
     const int slice = lane32 % LPR;
-    __shared__ float partial[2][kWaves][RPW];
-    float running = 0.0f;  // W2Accum: the row's sum so far (threads below RPW)
-    if (kAccum && threadIdx.x < RPW && row_block * RPW + threadIdx.x < a.N) {
-        running = a.out_f32[row_block * RPW + threadIdx.x];
-    }
+    const int row_blocks = a.N / RPW;
+    const int block_here = blockIdx.x * kWaves + wave;
+    const bool live_wave = block_here < row_blocks;          // a wave past the last row block still
+    const int row_block = live_wave ? block_here : row_blocks - 1;  // serves the copy and the barriers
+    const int row = row_block * RPW + row_in_block;
+    const bool writer = live_wave && half_id == 0 && slice == 0;
+    const int groups = a.iterations * LPR;
+    const int steps = (a.iterations + 1) / 2;
+    float running = 0.0f;  // W2Accum: the row's sum so far (writer lanes)
+    if (kAccum && writer) running = a.out_f32[row];
 
     for (int expert = first_expert; expert < last_expert; ++expert) {
     if (MODE == SwzMode::GateUp && expert == 0 && a.out_f32 != nullptr) {
@@ -82,7 +90,7 @@ __global__ __launch_bounds__(kWaves * 64) void swizzled_decode_kernel(SwzArgs a)
     if (kW2) {
         pa = static_cast<const uint4*>(a.w2.w2[expert]);
         sa = static_cast<const uint16_t*>(a.w2.s2[expert]);
-        x += static_cast<size_t>(expert) * (static_cast<size_t>(a.iterations) * LPR * 32);
+        x += static_cast<size_t>(expert) * (static_cast<size_t>(groups) * 32);
     } else {
         pa = static_cast<const uint4*>(a.w13.w1[expert]);
         sa = static_cast<const uint16_t*>(a.w13.s1[expert]);
@@ -92,15 +100,16 @@ __global__ __launch_bounds__(kWaves * 64) void swizzled_decode_kernel(SwzArgs a)
         }
     }
 
-    // Iterations owned by this lane: 2*wave + half_id, stepping by 2*kWaves.
+    // Step s of this lane is iteration 2s + half_id (the last step of an odd count has no
+    // second half: that lane reloads the last iteration and its product is dropped).
     const size_t block_base = static_cast<size_t>(row_block) * a.iterations * 32 + lane32;
-    uint4 wa[kMaxItersPerLane], wb[kMaxItersPerLane];
-    uint16_t ca[kMaxItersPerLane], cb[kMaxItersPerLane];
+    uint4 wa[kMaxSteps], wb[kMaxSteps];
+    uint16_t ca[kMaxSteps], cb[kMaxSteps];
+    auto fetch = [&](int first_step) {
 #pragma unroll
-    for (int j = 0; j < kMaxItersPerLane; ++j) {
-        const int it = 2 * wave + half_id + j * 2 * kWaves;
-        if (it < a.iterations) {
-            const size_t slot = block_base + static_cast<size_t>(it) * 32;
+        for (int j = 0; j < kMaxSteps; ++j) {
+            const int it = 2 * (first_step + j) + half_id;
+            const size_t slot = block_base + static_cast<size_t>(it < a.iterations ? it : a.iterations - 1) * 32;
             wa[j] = pa[slot];
             ca[j] = sa[slot];
             if (kTwo) {
@@ -108,18 +117,29 @@ __global__ __launch_bounds__(kWaves * 64) void swizzled_decode_kernel(SwzArgs a)
                 cb[j] = sb[slot];
             }
         }
+    };
+    fetch(0);   // in flight while the activations are copied
+
+    // the activation row into LDS, piece-major: x_lds[piece * groups + group]
+    const uint4* x4 = reinterpret_cast<const uint4*>(x);
+    for (int i = threadIdx.x; i < groups * 4; i += kWaves * 64) {
+        x_lds[(i & 3) * groups + (i >> 2)] = x4[i];
     }
+    __syncthreads();
 
     float acc_a = 0.0f, acc_b = 0.0f;
+    for (int first_step = 0; first_step < steps; first_step += kMaxSteps) {
+        if (first_step > 0) fetch(first_step);
 #pragma unroll
-    for (int j = 0; j < kMaxItersPerLane; ++j) {
-        const int it = 2 * wave + half_id + j * 2 * kWaves;
-        if (it < a.iterations) {
-            const int group = it * LPR + slice;
-            const uint4* xg = reinterpret_cast<const uint4*>(x + static_cast<size_t>(group) * 32);
-            uint4 xv[4] = {xg[0], xg[1], xg[2], xg[3]};
-            acc_a += half_bits_to_float(ca[j]) * group32_dot(wa[j], xv);
-            if (kTwo) acc_b += half_bits_to_float(cb[j]) * group32_dot(wb[j], xv);
+        for (int j = 0; j < kMaxSteps; ++j) {
+            const int it = 2 * (first_step + j) + half_id;
+            if (it < a.iterations) {
+                const int group = it * LPR + slice;
+                const uint4 xv[4] = {x_lds[group], x_lds[groups + group], x_lds[2 * groups + group],
+                                     x_lds[3 * groups + group]};
+                acc_a += half_bits_to_float(ca[j]) * group32_dot(wa[j], xv);
+                if (kTwo) acc_b += half_bits_to_float(cb[j]) * group32_dot(wb[j], xv);
+            }
         }
     }
 
@@ -127,43 +147,28 @@ __global__ __launch_bounds__(kWaves * 64) void swizzled_decode_kernel(SwzArgs a)
     acc_a = wave_xor_sum(acc_a, (LPR - 1) | 32);
     if (kTwo) acc_b = wave_xor_sum(acc_b, (LPR - 1) | 32);
 
-    if (half_id == 0 && slice == 0) {
-        partial[0][wave][row_in_block] = acc_a;
-        if (kTwo) partial[1][wave][row_in_block] = acc_b;
-    }
-    __syncthreads();
-
-    if (threadIdx.x < RPW) {
-        const int row = row_block * RPW + threadIdx.x;
-        float sum_a = 0.0f, sum_b = 0.0f;
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) {
-            sum_a += partial[0][w][threadIdx.x];
-            if (kTwo) sum_b += partial[1][w][threadIdx.x];
-        }
-        if (row < a.N) {
-            if (MODE == SwzMode::Gemv) {
-                a.out_a[row] = float_to_half_bits(sum_a);
-            } else if (MODE == SwzMode::Dual) {
-                a.out_a[row] = float_to_half_bits(sum_a);
-                a.out_b[row] = float_to_half_bits(sum_b);
-            } else if (MODE == SwzMode::GateUp) {
-                a.out_a[static_cast<size_t>(expert) * a.N + row] =
-                    float_to_half_bits(clamped_swiglu(sum_a, sum_b, a.limit));
-            } else if (MODE == SwzMode::W2Contrib) {
-                a.out_f32[static_cast<size_t>(expert) * a.N + row] = a.topk_weights[expert] * sum_a;
-            } else {
-                float contribution = a.topk_weights[expert] * sum_a;
-                if (expert == 0 && a.initial != nullptr) contribution += half_bits_to_float(a.initial[row]);
-                running += contribution;
-                if (expert == last_expert - 1) {
-                    a.out_f32[row] = running;
-                    a.out_a[row] = float_to_half_bits(running);
-                }
+    if (writer) {
+        if (MODE == SwzMode::Gemv) {
+            a.out_a[row] = float_to_half_bits(acc_a);
+        } else if (MODE == SwzMode::Dual) {
+            a.out_a[row] = float_to_half_bits(acc_a);
+            a.out_b[row] = float_to_half_bits(acc_b);
+        } else if (MODE == SwzMode::GateUp) {
+            a.out_a[static_cast<size_t>(expert) * a.N + row] =
+                float_to_half_bits(clamped_swiglu(acc_a, acc_b, a.limit));
+        } else if (MODE == SwzMode::W2Contrib) {
+            a.out_f32[static_cast<size_t>(expert) * a.N + row] = a.topk_weights[expert] * acc_a;
+        } else {
+            float contribution = a.topk_weights[expert] * acc_a;
+            if (expert == 0 && a.initial != nullptr) contribution += half_bits_to_float(a.initial[row]);
+            running += contribution;
+            if (expert == last_expert - 1) {
+                a.out_f32[row] = running;
+                a.out_a[row] = float_to_half_bits(running);
             }
         }
     }
-    if (kAccum) __syncthreads();  // the exchange buffer is reused by the next expert
+    if (kAccum) __syncthreads();  // the activation copy is replaced for the next expert
     }
 }
 
@@ -171,14 +176,19 @@ template <SwzMode MODE>
 static int launch(const SwzArgs& a, int rpw, int lpr, int experts, hipStream_t stream,
                   const char* who) {
     const dim3 block(kWaves * 64);
+    const size_t lds = static_cast<size_t>(a.iterations) * lpr * 64;  // K halves
+    auto grid = [&](int rows_per_block) {
+        const int row_blocks = a.N / rows_per_block;
+        return dim3((row_blocks + kWaves - 1) / kWaves, experts);
+    };
     if (rpw == 4 && lpr == 8) {
-        swizzled_decode_kernel<4, 8, MODE><<<dim3(a.N / 4, experts), block, 0, stream>>>(a);
+        swizzled_decode_kernel<4, 8, MODE><<<grid(4), block, lds, stream>>>(a);
     } else if (rpw == 8 && lpr == 4) {
-        swizzled_decode_kernel<8, 4, MODE><<<dim3(a.N / 8, experts), block, 0, stream>>>(a);
+        swizzled_decode_kernel<8, 4, MODE><<<grid(8), block, lds, stream>>>(a);
     } else if (rpw == 2 && lpr == 16) {
-        swizzled_decode_kernel<2, 16, MODE><<<dim3(a.N / 2, experts), block, 0, stream>>>(a);
+        swizzled_decode_kernel<2, 16, MODE><<<grid(2), block, lds, stream>>>(a);
     } else if (rpw == 16 && lpr == 2) {
-        swizzled_decode_kernel<16, 2, MODE><<<dim3(a.N / 16, experts), block, 0, stream>>>(a);
+        swizzled_decode_kernel<16, 2, MODE><<<grid(16), block, lds, stream>>>(a);
     } else {
         set_error("%s: unsupported swizzle geometry rpw=%d lpr=%d", who, rpw, lpr);
         return AEON_ERR_INVALID_ARGUMENT;
@@ -194,9 +204,8 @@ static int check_shape(int N, int K, int rpw, int lpr, const char* who) {
                  "%s: rpw*lpr must be 32 (rpw=%d lpr=%d)", who, rpw, lpr);
     AEON_REQUIRE(N > 0 && K > 0 && K % (lpr * 32) == 0 && N % rpw == 0, AEON_ERR_INVALID_ARGUMENT,
                  "%s: incompatible N/K shape (N=%d K=%d rpw=%d lpr=%d)", who, N, K, rpw, lpr);
-    AEON_REQUIRE(K / (lpr * 32) <= kMaxItersPerLane * 2 * kWaves, AEON_ERR_INVALID_ARGUMENT,
-                 "%s: K=%d exceeds the kernel's capacity of %d columns at lpr=%d", who, K,
-                 kMaxItersPerLane * 2 * kWaves * lpr * 32, lpr);
+    AEON_REQUIRE(K <= 32768, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: K=%d exceeds the 32768 columns whose activations fit the kernel's LDS copy", who, K);
     return AEON_OK;
 }
 
