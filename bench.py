@@ -161,6 +161,42 @@ def run_dropin(capi, moe, torch, np):
     ms = a.elapsed_time(b) / 320
     res["token_trio"] = {"ms_per_token": round(ms, 4),
                          "weights_gbps": round(K * expert_bytes / ms / 1e6, 1)}
+    # the single GEMV and dual GEMV entry points: the reference's shape and BASELINE config 0's,
+    # 64 launches on different matrices captured into one graph (a launch is shorter than a call)
+    res["gemv"] = []
+    for cols in (H, 7168):
+        mats = [(words(I * cols // 8), scales(I * cols // 32)) for _ in range(16)]
+        xv = (torch.rand(cols, device="cuda") - 0.5).half()
+        ya = torch.zeros(I, dtype=torch.float16, device="cuda")
+        yb = torch.zeros(I, dtype=torch.float16, device="cuda")
+        for dual in (False, True):
+            def one(i):
+                pa, sa = mats[i % 16]
+                pb, sb = mats[(i + 1) % 16]
+                if dual:
+                    capi.call("aeon_w4a16_swizzled_dual_gemv", capi.vp(xv), capi.vp(pa), capi.vp(sa),
+                              capi.vp(pb), capi.vp(sb), capi.vp(ya), capi.vp(yb), I, cols, 4, 8, sp())
+                else:
+                    capi.call("aeon_w4a16_swizzled_gemv", capi.vp(xv), capi.vp(pa), capi.vp(sa),
+                              capi.vp(ya), I, cols, 4, 8, sp())
+            one(0)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for i in range(64):
+                    one(i)
+            graph.replay()
+            torch.cuda.synchronize()
+            a.record()
+            for _ in range(5):
+                graph.replay()
+            b.record()
+            torch.cuda.synchronize()
+            us = a.elapsed_time(b) / (5 * 64) * 1e3
+            nbytes = (2 if dual else 1) * (I * cols // 2 + I * cols // 32 * 2)
+            res["gemv"].append({"N": I, "K": cols, "dual": dual, "us": round(us, 2),
+                                "gbps": round(nbytes / us / 1e3, 1)})
+        del mats
     res["chunks"] = []
     for T in (64, 256, 1024):
         rng = np.random.default_rng(T)
