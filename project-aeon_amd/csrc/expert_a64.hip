@@ -210,7 +210,7 @@ __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegD
         const int id = s == seg.slot_shared ? seg.slot_experts : seg.expert[s];
         if (id < 0 || (id >= seg.slot_experts && s != seg.slot_shared)) return;
         first = s;
-        count = 1;
+        count = s == seg.slot_shared ? seg.slot_tokens : 1;
         e = (GATE_UP ? gu.experts : dn.experts)[id];
     }
 
@@ -236,7 +236,8 @@ __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegD
     const int position = first + (n < count ? n : count - 1);
     const AEON_GLOBAL uint16_t* xrow;
     if (GATE_UP) {
-        const long row = slot_mode ? 0 : gu.row_index != nullptr ? gu.row_index[position] : position;
+        const long row = slot_mode ? (s == seg.slot_shared ? position - first : s / seg.slot_top_k)
+                         : gu.row_index != nullptr ? gu.row_index[position] : position;
         xrow = as_global<uint16_t>(gu.x) + row * gu.x_stride + chunk * 8;
     } else {
         xrow = as_global<uint16_t>(dn.hidden) + static_cast<size_t>(position) * dn.I + chunk * 8;
@@ -389,7 +390,7 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
     // slot mode (single token, no segment list): segment s is slot s of the caller's ids
     const bool slot_mode = seg.total == nullptr;
     const int first = slot_mode ? s : seg.first[s];
-    const int count = slot_mode ? 1 : seg.count[s];
+    const int count = slot_mode ? (s == seg.slot_shared ? seg.slot_tokens : 1) : seg.count[s];
     const int id = slot_mode && s == seg.slot_shared ? seg.slot_experts : seg.expert[s];
     const aeon_a64_expert e = (GATE_UP ? gu.experts : dn.experts)[id];
 
@@ -418,7 +419,8 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
         const int token = mt * kSegTokens + n;
         const int position = first + (token < count ? token : count - 1);
         if (GATE_UP) {
-            const long row = slot_mode ? 0 : gu.row_index != nullptr ? gu.row_index[position] : position;
+            const long row = slot_mode ? (s == seg.slot_shared ? position - first : s / seg.slot_top_k)
+                             : gu.row_index != nullptr ? gu.row_index[position] : position;
             xrow[mt] = as_global<uint16_t>(gu.x) + row * gu.x_stride + chunk * 8 + wave * 32;
         } else {
             xrow[mt] = as_global<uint16_t>(dn.hidden) + static_cast<size_t>(position) * dn.I + chunk * 8 +
@@ -583,7 +585,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const SegmentList& seg = GATE_UP ? gu.seg : dn.seg;
     const int s = blockIdx.y;  // the list is ordered costliest first
     if (seg.total == nullptr) {
-        // slot mode: one token, segment s = slot s; a dropped id ends the workgroup
+        // slot mode: segment s = draw s of a handful of tokens; a dropped id ends the workgroup
         if (s != seg.slot_shared) {
             const int id = seg.expert[s];
             if (id < 0 || id >= seg.slot_experts) return;

@@ -21,12 +21,15 @@ struct SegmentList {
     const int* total;   // [1] number of live segments (device); null = "direct" mode: one
                         // segment, positions 0..direct_count-1 of direct_expert
     int capacity;       // grid bound: blocks past *total exit at once
-    // "slot" mode for a single token (total == null, slot_experts > 0): segment s is the
-    // token's slot s -- expert[s] is read straight from the caller's top-k ids, position s,
-    // one token; an id outside [0, slot_experts) ends the workgroup. Segment `slot_shared`
-    // (if >= 0) is the always-on expert, table entry slot_experts, weight 1.
+    // "slot" mode for a handful of tokens (total == null, slot_experts > 0): segment s is draw
+    // s -- expert[s] is read straight from the caller's top-k ids [tokens][slot_top_k], position
+    // s, one token (row s / slot_top_k); an id outside [0, slot_experts) ends the workgroup.
+    // Segment `slot_shared` (if >= 0) is the always-on expert over all slot_tokens tokens: table
+    // entry slot_experts, weight 1, positions slot_shared..slot_shared+slot_tokens-1.
     int slot_experts;
     int slot_shared;
+    int slot_top_k;
+    int slot_tokens;   // <= kSegTokens
 };
 
 struct SegGateUpArgs {

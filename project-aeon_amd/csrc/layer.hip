@@ -15,6 +15,8 @@ namespace aeon355 {
 
 // Up to this many tokens a step is a decode batch; above it, a prefill chunk.
 constexpr int kDecodeMaxTokens = 128;
+// Up to this many tokens the expert kernels read the top-k ids directly (no permutation).
+constexpr int kSlotTokens = 2;
 
 static size_t align_up(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
 
@@ -176,10 +178,13 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
                      "%s: a chunk of %d tokens at this shape exceeds the 4 GiB the grouped kernels "
                      "address; split the chunk", who, tokens);
     }
-    // A single token needs no permutation: slot s of its top-k is segment s, read by the
-    // kernels straight from the caller's ids and weights (the always-on expert, if any, is one
-    // more segment), and its contribution rows are already in draw order.
-    const bool slots_direct = tokens == 1;
+    // A handful of tokens need no permutation: draw s of the top-k ids is segment s, read by
+    // the kernels straight from the caller's ids and weights (the always-on expert, if any, is
+    // one more segment over all tokens), and the contribution rows are already in draw order.
+    // An expert two of the tokens share is streamed twice that way: with a router that
+    // concentrates its choices that outweighs the saved launch from three tokens on (measured),
+    // so the limit is two.
+    const bool slots_direct = tokens <= kSlotTokens;
     if ((stage_mask & AEON_STAGE_PERMUTATION) && !slots_direct) {
         if (int rc = launch_permutation(p, s)) return rc;
     }
@@ -189,11 +194,11 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     gu.x_stride = x_stride;
     gu.row_index = w.token_indices;
     gu.experts = layer->d_experts;
-    gu.seg = SegmentList{w.seg_expert, w.seg_first, w.seg_count, w.seg_total, p.seg_capacity, 0, -1};
+    gu.seg = SegmentList{w.seg_expert, w.seg_first, w.seg_count, w.seg_total, p.seg_capacity, 0, -1, 0, 0};
     if (slots_direct) {
         gu.seg = SegmentList{d_topk_ids, nullptr, nullptr, nullptr,
-                             layer->top_k + (layer->has_shared ? 1 : 0), layer->experts,
-                             layer->has_shared ? layer->top_k : -1};
+                             draws + (layer->has_shared ? 1 : 0), layer->experts,
+                             layer->has_shared ? draws : -1, layer->top_k, tokens};
         gu.row_index = nullptr;
     }
     gu.hidden = w.hidden;

@@ -294,30 +294,39 @@ def test_out_of_range_ids_contribute_nothing(orc, T):
 
 
 @pytest.mark.parametrize("shared", [True, False])
-def test_single_token_reads_its_slots_directly(orc, shared):
-    """One token takes no permutation launch: the kernels read its ids and weights as they are.
-    Its result has to be the one the same token gets as row 0 of a two-token batch (which goes
-    through the permutation), bit for bit -- same kernels, same summation order -- and the
-    oracle's; without an always-on expert the routed sum is added to what the output holds."""
+def test_few_tokens_read_their_slots_directly(orc, shared):
+    """One or two tokens take no permutation launch: the kernels read the ids and weights as they
+    are, one segment per draw (tokens 0 and 1 share expert 2 here, which is then streamed twice).
+    A token's result has to be the one it gets in a six-token batch, which goes through the
+    permutation (to summation order: the two may pick different kernel forms), bit for bit the
+    one it gets alone, and the oracle's; without an always-on expert the routed sum is added to
+    what the output holds."""
     torch, h, capi, moe, synth = _setup()
     H, I, E, k, limit = 512, 384, 10, 4, 7.0
     pool = moe.ExpertPool(E + (1 if shared else 0), H, I)
     assert pool.fill_synthetic(seed=33, first_expert_id=0) == 0
     layer = moe.MoeLayer(pool, E, k, shared, limit)
-    ids = np.array([[7, 2, 9, 0], [1, 2, 3, 4]], dtype=np.int32)
-    w = synth.route_weights(33, 2 * k).reshape(2, k).astype(np.float32)
-    x = synth.activations(33, 2, H)
+    ids = np.array([[7, 2, 9, 0], [1, 2, 3, 4], [5, 6, 7, 8], [9, 8, 1, 0], [3, 5, 7, 9], [0, 2, 4, 6]],
+                   dtype=np.int32)
+    T = ids.shape[0]
+    w = synth.route_weights(33, T * k).reshape(T, k).astype(np.float32)
+    x = synth.activations(33, T, H)
     d_x, d_ids, d_w = h.dev_half(x), h.to_dev(ids), h.to_dev(w)
-    start = synth.activations(34, 2, H).astype(np.float16)
-    pair = layer.routed(d_x, d_ids, d_w, out=h.to_dev(start.copy())).cpu().numpy()
-    one = layer.routed(d_x[:1], d_ids[:1], d_w[:1], out=h.to_dev(start[:1].copy())).cpu().numpy()
-    assert np.array_equal(one[0], pair[0])
-    experts = {int(e): h.Expert(33, int(e), H, I) for e in ids[0]}
+    start = synth.activations(34, T, H).astype(np.float16)
+    six = layer.routed(d_x, d_ids, d_w, out=h.to_dev(start.copy())).cpu().numpy()
+    experts = {int(e): h.Expert(33, int(e), H, I) for e in np.unique(ids[:4])}
     sh = h.Expert(33, E, H, I) if shared else None
-    want = _oracle_layer(orc, h, experts, x[:1], ids[:1], w[:1], sh, limit)[0]
+    want = _oracle_layer(orc, h, experts, x[:4], ids[:4], w[:4], sh, limit)
     if not shared:
-        want = want + start[0].astype(np.float64)
-    assert np.abs(one[0] - want).max() <= 6e-3 * np.abs(want).max()
+        want = want + start[:4].astype(np.float64)
+    alone = [layer.routed(d_x[t:t + 1], d_ids[t:t + 1], d_w[t:t + 1],
+                          out=h.to_dev(start[t:t + 1].copy())).cpu().numpy()[0] for t in range(4)]
+    for n in (1, 2, 3, 4):
+        got = layer.routed(d_x[:n], d_ids[:n], d_w[:n], out=h.to_dev(start[:n].copy())).cpu().numpy()
+        assert np.abs(got - want[:n]).max() <= 6e-3 * np.abs(want).max(), n
+        assert np.abs(got - six[:n]).max() <= 1e-3 * np.abs(six).max(), n
+        for t in range(n):
+            assert np.array_equal(got[t], alone[t]), (n, t)
 
 
 def test_decode_segments_of_two_token_tiles(orc):
