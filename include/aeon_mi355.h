@@ -275,7 +275,9 @@ int aeon_moe_layer_routed(const aeon_moe_layer* layer, const void* d_x, int x_st
 
 /* The same step cut into its launches, for measurement: runs only the stages named in
  * stage_mask, on the state earlier stages left in the workspace (so AEON_STAGE_GATE_UP alone
- * can be repeated between two events once a full step has run with the same arguments). */
+ * can be repeated between two events once a full step has run with the same arguments). With
+ * one or two tokens the permutation stage launches nothing: the expert stages read the ids and
+ * weights directly. */
 #define AEON_STAGE_PERMUTATION 1
 #define AEON_STAGE_GATE_UP 2
 #define AEON_STAGE_DOWN 4
