@@ -234,6 +234,9 @@ def test_config2_full_size_sampled(orc):
     for t in (5, 40):
         alone = layer.routed(d_x[t:t + 1], ids_t[t:t + 1], w_t[t:t + 1]).cpu().numpy()
         assert np.abs(alone[0] - out[t]).max() <= 1e-3 * np.abs(out[t]).max()
+    # two tokens: one segment per draw, the always-on expert over both, wide W2 launch
+    pair = layer.routed(d_x[40:42], ids_t[40:42], w_t[40:42]).cpu().numpy()
+    assert np.abs(pair - out[40:42]).max() <= 1e-3 * np.abs(out[40:42]).max()
 
 
 @pytest.mark.parametrize("H,I,B", [(256, 128, 3), (256, 384, 5), (768, 256, 17), (256, 128, 70),
