@@ -4,6 +4,12 @@
 // are the reference's for hidden 4096 / intermediate 2048
 // (src/backend/swizzled_w4a16/core/swizzled_expert_format.hpp:9-30); swizzled_expert_layout()
 // states the same order for any shape.
+//
+// The kernels never take these offsets themselves: a caller (the reference's pool views, or
+// V4ResidentExpertPool here) adds them to an expert's base address and hands the six resulting
+// pointers to the weight tables. The device repack reads a payload through the same offsets
+// (aeon_payload_layout_for gives them for any hidden/intermediate pair) and writes the wave64
+// packing next to it, which has its own sub-tensor order (W1, W3, W2) and scale granularity.
 #include "infrastructure/expert/storage/expert_format.hpp"
 
 #include <cstddef>

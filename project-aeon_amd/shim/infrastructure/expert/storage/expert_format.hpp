@@ -2,6 +2,15 @@
 // Identity of an expert payload format under the reference's names
 // (src/infrastructure/expert/storage/expert_format.hpp:10-66). A loader compares an artifact's
 // header with one of these descriptors before it trusts any offset in the file.
+//
+// How the pieces are used on this path: the expert container's index file opens with a header
+// (magic, artifact version, layer count, experts per layer, payload bytes) followed by one
+// (offset, length) pair per expert; the reader (aeon_expert_catalog_open in the library,
+// V4ResidentExpertPool above it) accepts the file only if that header equals the descriptor
+// returned by make_current_swizzled_expert_format() for the same layer and expert counts, if
+// every payload starts on a sector boundary and is payload_bytes long, and if the catalog's size
+// arithmetic cannot overflow. The checks live here so that the writer's and the reader's idea of
+// "a valid catalog" is one piece of code.
 #include <cstddef>
 #include <cstdint>
 #include <limits>
