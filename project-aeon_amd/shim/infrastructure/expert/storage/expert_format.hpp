@@ -3,14 +3,13 @@
 // (src/infrastructure/expert/storage/expert_format.hpp:10-66). A loader compares an artifact's
 // header with one of these descriptors before it trusts any offset in the file.
 //
-// How the pieces are used on this path: the expert container's index file opens with a header
-// (magic, artifact version, layer count, experts per layer, payload bytes) followed by one
-// (offset, length) pair per expert; the reader (aeon_expert_catalog_open in the library,
-// V4ResidentExpertPool above it) accepts the file only if that header equals the descriptor
-// returned by make_current_swizzled_expert_format() for the same layer and expert counts, if
-// every payload starts on a sector boundary and is payload_bytes long, and if the catalog's size
-// arithmetic cannot overflow. The checks live here so that the writer's and the reader's idea of
-// "a valid catalog" is one piece of code.
+// On this path: the expert container's index file opens with a header (magic, artifact
+// version, layer count, experts per layer, payload bytes) followed by one (offset, length) pair
+// per expert. The library's reader (aeon_expert_catalog_open) applies the rules below in C --
+// version 2, a power-of-two sector, every payload on a sector boundary and payload_bytes long,
+// at least one layer and one expert, sizes that cannot overflow -- and this header gives C++
+// callers of the reference the descriptor type and the constants they compile against, with the
+// same rules as member functions.
 #include <cstddef>
 #include <cstdint>
 #include <limits>
