@@ -198,7 +198,10 @@ def run_dropin(capi, moe, torch, np):
                                 "gbps": round(nbytes / us / 1e3, 1)})
         del mats
     res["chunks"] = []
-    for T in (64, 256, 1024):
+    for T, NE in ((64, 64), (256, 64), (1024, 64), (256, 256)):
+        while len(experts) < NE:   # the reference's own layer: 256 experts, chunks of 256 tokens
+            experts.append({name: (words(r * c // 8), scales(r * c // 32))
+                            for name, r, c in (("w1", I, H), ("w3", I, H), ("w2", H, I))})
         rng = np.random.default_rng(T)
         ids_h = np.stack([rng.permutation(NE)[:K] for _ in range(T)]).astype(np.int32)
         ids = torch.from_numpy(ids_h).cuda()
@@ -235,7 +238,8 @@ def run_dropin(capi, moe, torch, np):
         b.record()
         torch.cuda.synchronize()
         ms = a.elapsed_time(b) / 20
-        res["chunks"].append({"tokens": T, "tokens_per_expert": round(draws / NE, 1),
+        res["chunks"].append({"tokens": T, "experts": NE, "tokens_per_expert": round(draws / NE, 1),
+                              "weights_gbps": round(NE * expert_bytes / ms / 1e6, 1),
                               "ms": round(ms, 3),
                               "tflops": round(2.0 * draws * 3 * H * I / ms / 1e9, 1)})
     return res

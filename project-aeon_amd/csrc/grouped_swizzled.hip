@@ -44,7 +44,7 @@ constexpr int kSwzWindowTiles = 4;  // token tiles of 16 positions one workgroup
 // wave fetches one step's activation fragments (j = its index) a group ahead and all four read
 // them from LDS: one barrier per 128 columns, two LDS buffers (the one written in pass G was
 // last read in pass G-1, before that pass's barrier). Weights and scales wait in a register
-// ring three passes deep.
+// ring three passes deep, six for windows of one or two token tiles.
 template <int RPW, int LPR, bool GATE_UP, int MT>
 __device__ __forceinline__ void grouped_swizzled_window(const GroupedSwzArgs& a, int expert, int first,
                                                         int count, int m0, half8_t* xs) {
@@ -107,7 +107,13 @@ __device__ __forceinline__ void grouped_swizzled_window(const GroupedSwzArgs& a,
     // Ring of kDepth passes of weights and scales in registers. Requests are kept in one order
     // everywhere (the next activation fragments, then the weights kDepth passes ahead): the
     // compiler's wait counts are static, so the order before the loop has to be the loop's.
-    constexpr int kDepth = 3;
+    // A window of one or two token tiles is bound by its weight stream and has registers to
+    // spare: its ring is twice as deep, and its activation fragments are fetched as far ahead
+    // as its weights. Loads land in issue order, so a fragment fetched only one pass ahead makes
+    // every older weight request land by the end of each pass and leaves two passes in flight
+    // whatever the ring's depth; the larger windows, whose passes are long, keep that form.
+    constexpr int kDepth = MT <= 2 ? 6 : 3;
+    constexpr int kAhead = MT <= 2 ? kDepth : 1;   // divides kDepth: pass G's slot is G % kAhead
     uint4 wa4[kDepth], wb4[kDepth];
     uint16_t s_a[kDepth], s_b[kDepth];
     auto fetch_weights = [&](int d, int G) {
@@ -122,14 +128,21 @@ __device__ __forceinline__ void grouped_swizzled_window(const GroupedSwzArgs& a,
             s_b[d] = 0;
         }
     };
-    half8_t xr[MT];
+    half8_t xr[kAhead][MT];   // xr[P % kAhead]: this wave's fragments of pass P
+    auto fetch_x = [&](int slot, int G) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) xr[slot][mt] = x_fragment(mt, G < passes ? G : passes - 1);
+    };
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) *lds(0, mt, wave) = x_fragment(mt, 0);
+    // the requests before the loop go out in the loop's order (the fragments a pass fetches,
+    // then the weights it fetches): the compiler's wait counts are static
 #pragma unroll
     for (int d = 0; d < kDepth; ++d) {
-        if (d == kDepth - 1) {
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) xr[mt] = x_fragment(mt, passes > 1 ? 1 : 0);
+        if (kAhead == kDepth) {
+            fetch_x((d + 1) % kAhead, d + 1);
+        } else if (d == kDepth - 1) {
+            fetch_x(0, 1);
         }
         fetch_weights(d, d);
         __builtin_amdgcn_sched_barrier(0);
@@ -159,12 +172,11 @@ __device__ __forceinline__ void grouped_swizzled_window(const GroupedSwzArgs& a,
                 }
             }
         }
+        const int next_slot = kAhead == 1 ? 0 : (d + 1) % kAhead;
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) *lds((G + 1) & 1, mt, wave) = xr[mt];
-        const int after = G + 2 < passes ? G + 2 : passes - 1;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) xr[mt] = x_fragment(mt, after);
-        fetch_weights(d, G + kDepth);   // past the end: the last pass again, unused
+        for (int mt = 0; mt < MT; ++mt) *lds((G + 1) & 1, mt, wave) = xr[next_slot][mt];
+        fetch_x(next_slot, G + 1 + kAhead);   // past the end: the last pass again, unused
+        fetch_weights(d, G + kDepth);
         __syncthreads();
     };
     int G0 = 0;
