@@ -695,14 +695,26 @@ __global__ __launch_bounds__(256) void token_reduce_kernel(
         for (int q = 0; q < 4; ++q) acc[q] = half_bits_to_float(initial[t * initial_stride + i + q]);
     }
     const float* c = contrib + static_cast<size_t>(t) * slots * hidden + i;
-    for (int s = 0; s < slots; ++s) {
-        if (ids != nullptr) {
-            const int e = ids[t * slots + s];
-            if (e < 0 || e >= experts) continue;
-        }
-        const float4_t v = *reinterpret_cast<const float4_t*>(c + static_cast<size_t>(s) * hidden);
+    // Eight slots at a time: their rows are requested first, whether they count or not (a
+    // dropped slot's row is stale but addressable), so that no request waits for an id; the ids
+    // only decide which of the loaded rows are added, in slot order.
+    for (int s0 = 0; s0 < slots; s0 += 8) {
+        float4_t v[8];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) acc[q] += v[q];
+        for (int j = 0; j < 8; ++j) {
+            const int s = s0 + j < slots ? s0 + j : slots - 1;
+            v[j] = *reinterpret_cast<const float4_t*>(c + static_cast<size_t>(s) * hidden);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (s0 + j >= slots) break;
+            if (ids != nullptr) {
+                const int e = ids[t * slots + s0 + j];
+                if (e < 0 || e >= experts) continue;
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc[q] += v[j][q];
+        }
     }
     uint16_t* o = out + t * out_stride + i;
     if ((reinterpret_cast<uintptr_t>(o) & 7) == 0) {
