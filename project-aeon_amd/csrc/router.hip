@@ -188,7 +188,7 @@ __global__ __launch_bounds__(256 * kParts) void router_topk_kernel(
 
     const bool hashed = hash_table != nullptr && token_ids != nullptr;
     if (hashed) {
-        if (threadIdx.x < top_k) {
+        if (static_cast<int>(threadIdx.x) < top_k) {
             const int e = static_cast<int>(
                 hash_table[static_cast<size_t>(token_ids[token]) * top_k + threadIdx.x]);
             picked_id[threadIdx.x] = e;
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(256 * kParts) void router_topk_kernel(
         }
     }
     __syncthreads();
-    if (threadIdx.x < top_k) {
+    if (static_cast<int>(threadIdx.x) < top_k) {
         double sum = 0.0;
         for (int k = 0; k < top_k; ++k) sum += picked_score[k];
         double w = picked_score[threadIdx.x];
