@@ -210,3 +210,42 @@ def test_resident_load_counts_unequal_scales(tmp_path, experts):
         assert pool.load_catalog(cat, 1) == 0
     finally:
         capi.lib().aeon_expert_catalog_close(cat)
+
+
+def test_catalog_reader_survives_mutated_indexes_under_host_sanitizers(tmp_path):
+    """The reader parses a file it has no reason to trust. Its source file is rebuilt with the
+    host-side address and undefined-behaviour sanitizers (device code untouched), linked into a
+    driver that feeds it mutated index files, and the driver has to end normally: every mutation
+    either rejected or opened, read and closed without a sanitizer finding."""
+    import shutil
+    import subprocess
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not available")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    csrc = os.path.join(root, "project-aeon_amd", "csrc")
+    lib_dir = os.path.join(root, "project-aeon_amd")
+    if not os.path.exists(os.path.join(lib_dir, "libaeon_mi355.so")):
+        pytest.skip("library not built")
+    inc = ["-I", os.path.join(root, "include"), "-I", csrc]
+    dev = ["--offload-arch=gfx950", "-O1", "-g", "-std=c++17", "-fPIC", "-Xclang", "-target-feature",
+           "-Xclang", "-packed-fp32-ops"]
+    san = ["-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined",
+           "-Xarch_host", "-fno-sanitize-recover=undefined"]
+    objs = []
+    for src, extra in (("artifact.hip", []), ("errors.cpp", ["-x", "hip"])):
+        obj = str(tmp_path / (src + ".o"))
+        subprocess.run([hipcc] + dev + san + extra + inc + ["-c", os.path.join(csrc, src), "-o", obj],
+                       check=True, capture_output=True)
+        objs.append(obj)
+    driver = str(tmp_path / "fuzz.o")
+    subprocess.run([hipcc] + dev + san + ["-x", "hip"] + inc + ["-c",
+                    os.path.join(root, "tests", "cpp", "fuzz_catalog.cpp"), "-o", driver],
+                   check=True, capture_output=True)
+    exe = str(tmp_path / "fuzz_catalog")
+    subprocess.run([hipcc, "--offload-arch=gfx950", "-fsanitize=address,undefined", "-fno-gpu-sanitize",
+                    driver] + objs + ["-L", lib_dir, "-laeon_mi355", "-Wl,-rpath," + lib_dir, "-o", exe],
+                   check=True, capture_output=True)
+    run = subprocess.run([exe, "4000"], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert "opened" in run.stdout and "rejected" in run.stdout
