@@ -89,3 +89,37 @@ def test_a64_repack_rejects_unequal_group32_scales(orc):
         capi.call("aeon_a64_repack_host", u32p(swp), u16p(sws), N, K, 4, 8, u32p(out_p), u16p(out_s))
     with pytest.raises(ValueError):
         capi.call("aeon_a64_repack_host", u32p(swp), u16p(sws), 8, 256, 4, 8, u32p(out_p), u16p(out_s))
+
+
+def test_host_layout_functions_under_host_sanitizers(tmp_path):
+    """Swizzle / unswizzle and the wave64 repack / unrepack on exact-size heap buffers, with the
+    layout source file rebuilt under the host-side address and undefined-behaviour sanitizers
+    (device code untouched): an access one element past an end, or an overflowing index, ends the
+    driver; it also checks both round trips."""
+    import os
+    import shutil
+    import subprocess
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    csrc = os.path.join(root, "project-aeon_amd", "csrc")
+    lib_dir = os.path.join(root, "project-aeon_amd")
+    if not os.path.exists(hipcc) or not os.path.exists(os.path.join(lib_dir, "libaeon_mi355.so")):
+        pytest.skip("hipcc or the library is not available")
+    inc = ["-I", os.path.join(root, "include"), "-I", csrc]
+    dev = ["--offload-arch=gfx950", "-O1", "-g", "-std=c++17", "-fPIC", "-Xclang", "-target-feature",
+           "-Xclang", "-packed-fp32-ops"]
+    san = ["-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined",
+           "-Xarch_host", "-fno-sanitize-recover=undefined"]
+    objs = []
+    for src, extra in ((os.path.join(csrc, "layout.hip"), []), (os.path.join(csrc, "errors.cpp"), ["-x", "hip"]),
+                       (os.path.join(root, "tests", "cpp", "layout_asan.cpp"), ["-x", "hip"])):
+        obj = str(tmp_path / (os.path.basename(src) + ".o"))
+        subprocess.run([hipcc] + dev + san + extra + inc + ["-c", src, "-o", obj], check=True,
+                       capture_output=True)
+        objs.append(obj)
+    exe = str(tmp_path / "layout_asan")
+    subprocess.run([hipcc, "--offload-arch=gfx950", "-fsanitize=address,undefined", "-fno-gpu-sanitize"]
+                   + objs + ["-L", lib_dir, "-laeon_mi355", "-Wl,-rpath," + lib_dir, "-o", exe],
+                   check=True, capture_output=True)
+    run = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0 and run.stdout.strip().endswith("ok"), run.stdout[-1000:] + run.stderr[-2000:]
