@@ -374,3 +374,37 @@ def test_swizzled_grouped_windows_against_oracle(orc):
         want = weights[:c, e].astype(np.float64)[:, None] * o
         got_c = got_contrib[rows].astype(np.float64)
         assert np.abs(got_c - want).max() <= 2e-3 * np.abs(want).max(), (e, c)
+
+
+def test_swizzled_gemv_random_shapes_all_geometries(orc):
+    """Forty-eight seeded shapes through the `.aeon`-layout GEMV and dual GEMV: the four storage
+    geometries, 1..40 iterations (odd counts, more steps than one lane keeps in flight), row block
+    counts that leave waves of the last workgroup without a block. Against the oracle's matvec at
+    1e-2; the dual call's first output equals the single call's bit for bit."""
+    torch, h, capi = _setup()
+    rng = np.random.default_rng(3)
+    for case in range(48):
+        rpw, lpr = [(4, 8), (8, 4), (2, 16), (16, 2)][case % 4]
+        K = int(rng.integers(1, 41)) * lpr * 32
+        N = rpw * int(rng.integers(1, 40))
+        mats = []
+        for _ in range(2):
+            packed = rng.integers(0, 2**32, N * K // 8, dtype=np.uint64).astype(np.uint32)
+            scale = (0.004 + 0.02 * rng.random(N * K // 32)).astype(np.float16).view(np.uint16)
+            mats.append((packed, scale))
+        x = rng.standard_normal(K).astype(np.float16)
+        d_x = h.dev_half(x)
+        dev = [(h.dev_u32(p), h.dev_u16(s_)) for p, s_ in mats]
+        y1 = torch.zeros(N, dtype=torch.float16, device="cuda")
+        ya, yb = torch.zeros_like(y1), torch.zeros_like(y1)
+        capi.call("aeon_w4a16_swizzled_gemv", capi.vp(d_x), capi.vp(dev[0][0]), capi.vp(dev[0][1]),
+                  capi.vp(y1), N, K, rpw, lpr, h.stream_ptr())
+        capi.call("aeon_w4a16_swizzled_dual_gemv", capi.vp(d_x), capi.vp(dev[0][0]), capi.vp(dev[0][1]),
+                  capi.vp(dev[1][0]), capi.vp(dev[1][1]), capi.vp(ya), capi.vp(yb), N, K, rpw, lpr,
+                  h.stream_ptr())
+        torch.cuda.synchronize()
+        what = (case, rpw, lpr, N, K)
+        assert torch.equal(y1, ya), what
+        for got, (p, s_) in ((ya, mats[0]), (yb, mats[1])):
+            want = orc.swizzled_matvec(p, s_, N, K, rpw, lpr, x.astype(np.float64)[None, :])[0]
+            assert h.rel_err(got.cpu().numpy(), want) <= TOL, what
