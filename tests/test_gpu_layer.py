@@ -525,3 +525,42 @@ def test_random_layer_steps_against_oracle(orc):
                 first = start[t].astype(np.float64)
             want = orc.moe_combine(contrib, first) if keep else first.astype(np.float16).astype(np.float64)
             assert np.abs(out[t] - want).max() <= 6e-3 * max(np.abs(want).max(), 1e-6), (what, t)
+
+
+@pytest.mark.parametrize("B", [1, 8, 150])
+def test_layer_step_replays_from_a_captured_graph(orc, B):
+    """The step allocates nothing, clears nothing with a memset and never synchronises, so it can
+    be recorded into a HIP graph: the graph is replayed four times with new activations copied
+    into its input buffer and eager work between the replays, and every replay has to give the
+    bits of the eager step on the same activations (direct slots, decode segments, grouped
+    windows)."""
+    torch, h, capi, moe, synth = _setup()
+    H, I, E, k, limit = 512, 256, 20, 4, 7.0
+    pool = moe.ExpertPool(E + 1, H, I)
+    assert pool.fill_synthetic(seed=61, first_expert_id=0) == 0
+    wr, bias = synth.router_weight(61, H, E), synth.router_bias(61, E)
+    layer = moe.MoeLayer(pool, E, k, True, limit, h.to_dev(wr), h.to_dev(bias), score_kind=1)
+    xs = [h.dev_half(synth.activations(61, B, H, unit=10 + r)) for r in range(4)]
+    eager = []
+    for x in xs:
+        out, ids, w = layer.decode(x)
+        eager.append((out.clone(), ids.clone(), w.clone()))
+    torch.cuda.synchronize()
+    x_in = xs[0].clone()
+    out = torch.empty(B, H, dtype=torch.float16, device="cuda")
+    ids = torch.empty(B, k, dtype=torch.int32, device="cuda")
+    w = torch.empty(B, k, dtype=torch.float32, device="cuda")
+    layer.decode(x_in, out, ids, w)          # warm: the workspace exists before the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        layer.decode(x_in, out, ids, w)
+    for r in (1, 0, 3, 2):
+        x_in.copy_(xs[r])
+        scratch = layer.routed(xs[(r + 1) % 4], eager[(r + 1) % 4][1], eager[(r + 1) % 4][2])  # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager[r][0]), (B, r)
+        assert torch.equal(ids, eager[r][1]) and torch.equal(w, eager[r][2]), (B, r)
+        del scratch
