@@ -44,7 +44,12 @@ __global__ __launch_bounds__(kRouterWaves * 64) void router_logits_partial_kerne
     constexpr int kSteps = kRouterWaveRows / 16;
     uint2 xa[kSteps];
     float4_t b[kSteps][4];
-    const bool whole = (e + 3 < experts) && (h_begin + kRouterWaveRows <= hidden) && (x_stride % 4 == 0);
+    // the fast path reads 16 bytes of a weight row at column e and 8 bytes of an activation row:
+    // both must be aligned, which an expert count that is not a multiple of four (rows of the
+    // weight then start at 4-byte offsets) or an odd base pointer would break
+    const bool whole = (e + 3 < experts) && (experts % 4 == 0) && (h_begin + kRouterWaveRows <= hidden) &&
+                       (x_stride % 4 == 0) && ((reinterpret_cast<uintptr_t>(wr) & 15) == 0) &&
+                       ((reinterpret_cast<uintptr_t>(x) & 7) == 0);
     if (whole) {
 #pragma unroll
         for (int step = 0; step < kSteps; ++step) {

@@ -1,8 +1,17 @@
 #pragma once
-// The routed-expert seam of the layer body: the V4RoutedExpertExecutor interface with the
-// reference's method names, argument meaning and defaults
-// (src/architecture/deepseek_v4/layer/v4_layer_body_moe.hpp:32-112). Only the seam is here; the
-// layer body that drives it stays the reference's.
+// The routed-expert seam of the layer body, src/architecture/deepseek_v4/layer/
+// v4_layer_body_moe.hpp:32-112.
+//
+// When the reference tree follows this directory on the include path, this file steps aside:
+// the reference's own header is taken whole (#include_next), so the layer body keeps
+// dispatch_router, run_layer_body_router, run_layer_body_moe_shared_expert,
+// run_layer_body_moe_post and run_layer_body_moe_and_post (:124-312) and its one definition of
+// V4RoutedExpertExecutor, and nothing is added to it. Built without the reference tree (the
+// gates of the resident executor), only the interface is declared here, with the reference's
+// method names, argument meaning and defaults.
+#if __has_include_next("architecture/deepseek_v4/layer/v4_layer_body_moe.hpp")
+#include_next "architecture/deepseek_v4/layer/v4_layer_body_moe.hpp"
+#else
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
@@ -58,3 +67,4 @@ public:
 };
 
 }  // namespace aeon::core
+#endif

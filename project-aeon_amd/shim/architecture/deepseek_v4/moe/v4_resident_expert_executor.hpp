@@ -28,12 +28,14 @@ public:
         if (layers_.empty() || max_tokens <= 0) {
             throw std::invalid_argument("V4ResidentExpertExecutor: no layers or no tokens");
         }
+        int widest_top_k = 0;
         for (aeon_moe_layer& layer : layers_) {
             layer.has_shared = 0;
+            widest_top_k = std::max(widest_top_k, layer.top_k);
             workspace_bytes_ = std::max(workspace_bytes_, aeon_moe_layer_workspace_bytes(&layer, max_tokens));
         }
         CHECK_HIP(hipMalloc(&workspace_, workspace_bytes_));
-        CHECK_HIP(hipMalloc(&d_ids_, sizeof(int32_t) * max_tokens * layers_[0].top_k));
+        CHECK_HIP(hipMalloc(&d_ids_, sizeof(int32_t) * max_tokens * widest_top_k));
     }
 
     ~V4ResidentExpertExecutor() override {

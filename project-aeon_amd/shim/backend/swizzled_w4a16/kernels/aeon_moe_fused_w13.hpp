@@ -4,6 +4,7 @@
 #include "backend/swizzled_w4a16/kernels/aeon_w4a16_swizzled_gemv.hpp"
 
 #include <cstring>
+#include <type_traits>
 
 namespace aeon::kernel {
 
@@ -18,15 +19,17 @@ struct SwizzledW13ExpertPtrs {
 static_assert(sizeof(SwizzledW13ExpertPtrs) == sizeof(aeon_w13_table),
               "the table is handed to the C ABI by layout");
 
-// The gate/up pair with the model's clamped SwiGLU. The reference takes any `Epilogue` functor;
-// the library implements the one the model uses.
-template <int WAVES, int RPW, int LPR, int ITERS>
+// The gate/up pair. `Epilogue` is a template parameter as in the reference (:113); the library
+// behind this call implements the model's clamped SwiGLU, so that is the one policy accepted --
+// any other is refused when the call is compiled, not computed with the wrong rule.
+template <int WAVES, int RPW, int LPR, int ITERS, class Epilogue>
 inline void dispatch_aeon_moe_fused_gate_up(const half* activation,
                                             const SwizzledW13ExpertPtrs& weights,
                                             half* expert_hidden, float* output_f32, int output_dim,
                                             int expert_count, int N, int K,
-                                            Dsv4ClampedSwiGLUEpilogue epilogue,
-                                            hipStream_t stream = 0) {
+                                            Epilogue epilogue, hipStream_t stream = 0) {
+    static_assert(std::is_same_v<Epilogue, Dsv4ClampedSwiGLUEpilogue>,
+                  "the gfx950 gate/up kernels implement Dsv4ClampedSwiGLUEpilogue only");
     static_assert(RPW * LPR == 32, "RPW and LPR must describe one 32-slot storage tile");
     if (expert_count <= 0 || expert_count > kAeonSwizzledMaxExperts || N <= 0 ||
         K != ITERS * LPR * 32 || N % RPW != 0) {

@@ -1,8 +1,13 @@
 #pragma once
 // Device selection for the gates that include this header (reference: src/platform/device.hpp:26-58,
-// aeon::core::select_device). Same contract: the index is validated against the visible devices
-// and made current, a bad index or a failing runtime call is a std::runtime_error naming the call,
-// never a silent fallback to another device.
+// aeon::core::select_device). With the reference tree behind this directory on the include path
+// the reference's own header is taken whole (it also carries DeviceScope, :64-84); without it,
+// select_device alone is provided under the same contract: the index is validated against the
+// visible devices and made current, a bad index or a failing runtime call is a
+// std::runtime_error naming the call, never a silent fallback to another device.
+#if __has_include_next("platform/device.hpp")
+#include_next "platform/device.hpp"
+#else
 #include <hip/hip_runtime.h>
 
 #include <iostream>
@@ -35,3 +40,4 @@ inline int select_device(int index, bool verbose = true) {
 }
 
 }  // namespace aeon::core
+#endif

@@ -14,7 +14,8 @@ BIN = os.path.join(HERE, "cpp", "bin")
 
 
 @pytest.mark.parametrize("gate", ["test_swizzled_gemv", "test_grouped_batch_parity",
-                                  "test_resident_executor", "test_resident_pool"])
+                                  "test_resident_executor", "test_resident_pool",
+                                  "test_elementwise_controls"])
 def test_cpp_gate(gate):
     path = os.path.join(BIN, gate)
     assert os.path.exists(path), "tests/cpp is not built: run __graft_entry__.build()"

@@ -408,3 +408,38 @@ def test_swizzled_gemv_random_shapes_all_geometries(orc):
         for got, (p, s_) in ((ya, mats[0]), (yb, mats[1])):
             want = orc.swizzled_matvec(p, s_, N, K, rpw, lpr, x.astype(np.float64)[None, :])[0]
             assert h.rel_err(got.cpu().numpy(), want) <= TOL, what
+
+
+def test_standalone_swiglu_clamp_against_the_oracle(orc):
+    """aeon_swiglu_clamp (v4_swiglu_clamp_kernel, kernels/v4_swiglu_clamp.hpp:18-34) against
+    orc.clamped_swiglu: every pair of the reference's probes {-40,-12,-5,0,5,12,40,3}
+    (tests/test_v4_expert_oracle.cpp:302-406: gate < -limit and |up| > limit included) at limits
+    7 and 10, then a seeded sweep whose length is not a multiple of the block size. The output
+    is one fp16 rounding of an fp32 evaluation: it must equal the fp16 rounding of the oracle's
+    fp64 value or its neighbour. The symmetric-clamp misreading (mode 1) must be far off on the
+    gate < -limit probes, so the comparison can tell the two rules apart."""
+    torch, h, capi = _setup()
+    probes = np.array([-40, -12, -5, 0, 5, 12, 40, 3], dtype=np.float16)
+    g, u = [a.ravel() for a in np.meshgrid(probes, probes, indexing="ij")]
+    rng = np.random.default_rng(77)
+    g = np.concatenate([g, rng.uniform(-15, 15, 5003).astype(np.float16)])
+    u = np.concatenate([u, rng.uniform(-15, 15, 5003).astype(np.float16)])
+    d_g, d_u = h.dev_half(g), h.dev_half(u)
+    for limit in (7.0, 10.0):
+        out = torch.full((g.size + 16,), 123.0, dtype=torch.float16, device="cuda")
+        capi.call("aeon_swiglu_clamp", capi.vp(d_g), capi.vp(d_u), capi.vp(out), g.size,
+                  C.c_float(limit), h.stream_ptr())
+        got = out.cpu().numpy()
+        assert np.all(got[g.size:] == np.float16(123.0))        # nothing written past the end
+        got = got[:g.size]
+        want = np.array([orc.clamped_swiglu(float(a), float(b), limit) for a, b in zip(g, u)])
+        want16 = want.astype(np.float16)
+        lo = np.nextafter(want16, np.float16(-np.inf))
+        hi = np.nextafter(want16, np.float16(np.inf))
+        assert np.all((got == want16) | (got == lo) | (got == hi))
+        assert np.mean(got == want16) > 0.97
+        wrong = np.array([orc.clamped_swiglu(float(a), float(b), limit, 1) for a, b in zip(g, u)])
+        edge = (g.astype(np.float64) < -limit) & (np.abs(u.astype(np.float64)) >= 3)
+        assert edge.sum() >= 10
+        assert np.all(np.abs(got[edge].astype(np.float64) - wrong[edge]) >
+                      0.5 * np.abs(wrong[edge]))

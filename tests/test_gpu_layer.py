@@ -99,6 +99,29 @@ def test_router_ids_bit_exact_on_identical_logits(orc, score_kind, k, scaling):
     assert np.array_equal(ids, table[tok].astype(np.int32))
 
 
+@pytest.mark.parametrize("T,H,E", [(5, 1024, 10), (33, 896, 6), (3, 7168, 258), (17, 200, 64)])
+def test_router_logits_at_expert_counts_not_divisible_by_four(orc, T, H, E):
+    """aeon_router_logits where a weight row is not a whole number of 16-byte vectors (E % 4 != 0)
+    or the hidden size is not a whole number of chunks: the aligned fast path must step aside.
+    Against the fp64 product; run twice for bit-reproducibility."""
+    torch, h, capi, moe, synth = _setup()
+    rng = np.random.default_rng(T * 1000 + E)
+    x = rng.normal(0, 1, (T, H)).astype(np.float16)
+    wr = rng.normal(0, 0.05, (H, E)).astype(np.float32)
+    d_x, d_wr = h.dev_half(x), h.to_dev(wr)
+    n = capi.lib().aeon_router_logits_workspace_bytes(T, H, E)
+    ws = torch.empty(max(n, 4), dtype=torch.uint8, device="cuda")
+    outs = []
+    for _ in range(2):
+        out = torch.full((T, E), 7.0, dtype=torch.float32, device="cuda")
+        capi.call("aeon_router_logits", capi.vp(d_x), H, capi.vp(d_wr), capi.vp(out), T, H, E,
+                  capi.vp(ws), C.c_size_t(ws.numel()), h.stream_ptr())
+        outs.append(out.cpu().numpy())
+    want = x.astype(np.float64) @ wr.astype(np.float64)
+    assert np.abs(outs[0] - want).max() <= 1e-5 * np.abs(want).max()
+    assert np.array_equal(outs[0], outs[1])
+
+
 @pytest.mark.parametrize("T,slots,E", [(1, 8, 256), (7, 6, 256), (300, 6, 256), (64, 8, 8),
                                        (0, 8, 256), (2048, 8, 256), (64, 8, 1024),
                                        (128, 8, 256), (129, 8, 256), (1024, 1, 3), (171, 6, 1024),
