@@ -76,7 +76,7 @@ int main() {
         const double tol = std::fabs(want) * 0.0010 + 6e-8;
         worst = std::fmax(worst, std::fabs(got - want) - tol);
         close = close && std::fabs(got - want) <= tol;
-        if (g < -limit) {
+        if (g <= -limit - 3.0f) {
             // the gate is NOT clamped from below: silu(g) of the raw gate, far from silu(-L)
             const float symmetric = clamp_definition(-limit, u, limit);
             if (std::fabs(u) >= 3.0f && std::fabs(symmetric) > 1e-3f) {
@@ -112,22 +112,30 @@ int main() {
         GATE_HIP(hipFree(d_out));
     }
     const std::vector<half> chained = to_host(d_accum, hidden);
-    // The definition leaves the product's rounding open (a compiler may fuse the multiply into
-    // the add): every element must equal the chain evaluated with or without that fusion at
-    // each step. Both candidate chains are tracked; a device that fuses consistently follows one.
+    // The definition leaves the roundings inside a step open: a compiler may keep the product and
+    // the sum apart (two fp32 roundings, then fp16), fuse them (one fp32 rounding, then fp16), or
+    // use the mixed-precision fused multiply-add that rounds the exact sum to fp16 directly
+    // (v_fma_mixlo_f16). Each reading is followed as a chain of its own; the kernel is compiled
+    // one way, so it follows one of them through all the experts.
     bool chain_ok = true;
     int differs_from_single_rounding = 0;
     for (int i = 0; i < hidden; ++i) {
-        float plain = __half2float(accum[i]), fused = plain;
+        float plain = __half2float(accum[i]), fused = plain, direct = plain;
         double exact = plain;
         for (int e = 0; e < experts; ++e) {
             const float x = __half2float(outs[e][i]);
             plain = __half2float(__float2half(plain + weights[e] * x));
             fused = __half2float(__float2half(std::fmaf(weights[e], x, fused)));
+            direct = static_cast<float>(static_cast<_Float16>(static_cast<double>(direct) +
+                                                              static_cast<double>(weights[e]) * x));
             exact += static_cast<double>(weights[e]) * x;
         }
         const float got = __half2float(chained[i]);
-        chain_ok = chain_ok && (got == plain || got == fused);
+        if (!(got == plain || got == fused || got == direct) && chain_ok) {
+            std::printf("    element %d: device %.9g, chains %.9g / %.9g / %.9g, exact %.9g\n", i, got,
+                        plain, fused, direct, exact);
+        }
+        chain_ok = chain_ok && (got == plain || got == fused || got == direct);
         if (got != __half2float(__float2half(static_cast<float>(exact)))) ++differs_from_single_rounding;
     }
     expect(chain_ok, "moe_accumulate_expert_kernel == the fp16 chain, one rounding per expert");

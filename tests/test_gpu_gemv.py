@@ -439,7 +439,7 @@ def test_standalone_swiglu_clamp_against_the_oracle(orc):
         assert np.all((got == want16) | (got == lo) | (got == hi))
         assert np.mean(got == want16) > 0.97
         wrong = np.array([orc.clamped_swiglu(float(a), float(b), limit, 1) for a, b in zip(g, u)])
-        edge = (g.astype(np.float64) < -limit) & (np.abs(u.astype(np.float64)) >= 3)
+        edge = (g.astype(np.float64) <= -limit - 3) & (np.abs(u.astype(np.float64)) >= 3)
         assert edge.sum() >= 10
         assert np.all(np.abs(got[edge].astype(np.float64) - wrong[edge]) >
                       0.5 * np.abs(wrong[edge]))
