@@ -296,6 +296,25 @@ int aeon_moe_layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, i
 int aeon_moe_layer_decode(const aeon_moe_layer* layer, const void* d_x, int x_stride, int tokens,
                           void* d_out, int out_stride, int32_t* d_topk_ids, float* d_topk_weights,
                           void* d_workspace, size_t workspace_bytes, void* stream);
+/* aeon_moe_layer_decode with no workspace argument and no allocation. It has no counterpart in
+ * the reference: it is for callers that cannot allocate device memory or carry a workspace --
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc. The
+ * workspace is a fixed array of AEON_NOALLOC_WORKSPACE_BYTES inside the library's code object
+ * (every GPU the library runs on holds one copy until the process ends); the call launches the
+ * same kernels as aeon_moe_layer_decode on it and calls no hipMalloc, hipFree, hipMemset or
+ * allocating library routine. The first call on a device looks the array's address up once
+ * (hipGetSymbolAddress, with that device current) and is best made before any capture.
+ * Limit: aeon_moe_layer_workspace_bytes(layer, tokens) <= AEON_NOALLOC_WORKSPACE_BYTES (batch 64
+ * at hidden 7168 / intermediate 2048 / top-8 of 256 experts + always-on expert needs 19.1 MiB);
+ * beyond it the call returns AEON_ERR_INVALID_ARGUMENT and launches nothing.
+ * All calls on one GPU share that GPU's array: two calls that overlap in time on one GPU (two
+ * streams, two threads) race and must be serialised by the caller. Nothing in the array has to
+ * start at zero -- every word a kernel of the step reads was written earlier in the same step --
+ * so a call is not affected by what the previous one left behind. */
+#define AEON_NOALLOC_WORKSPACE_BYTES (24u << 20)
+int aeon_moe_layer_decode_noalloc(const aeon_moe_layer* layer, const void* d_x, int x_stride,
+                                  int tokens, void* d_out, int out_stride, int32_t* d_topk_ids,
+                                  float* d_topk_weights, void* stream);
 /* Device pointer to the fp32 logits [tokens][experts] the last aeon_moe_layer_decode call with
  * this workspace and token count left behind (what the ids were selected from). */
 const float* aeon_moe_layer_logits(const aeon_moe_layer* layer, int tokens, void* d_workspace);

@@ -8,6 +8,7 @@
 #include "router.hpp"
 
 #include <cstdlib>
+#include <mutex>
 
 extern "C" size_t aeon_router_logits_workspace_bytes(int tokens, int hidden, int experts);
 
@@ -289,6 +290,65 @@ extern "C" int aeon_moe_layer_decode(const aeon_moe_layer* layer, const void* d_
     }
     return aeon_moe_layer_routed(layer, d_x, x_stride, tokens, d_topk_ids, d_topk_weights, d_out,
                                  out_stride, d_workspace, workspace_bytes, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The step without an allocation anywhere: the workspace is a fixed array in device memory
+// ---------------------------------------------------------------------------------------------
+
+// The workspace of aeon_moe_layer_decode_noalloc. Each GPU the library runs on holds its own
+// copy of this array, at its own address, from the moment the code object is loaded until the
+// process ends. In host code the name below is only a handle for hipGetSymbolAddress: the
+// kernels are given the address that call returns, never the name.
+static __device__ __align__(256) unsigned char scratch[AEON_NOALLOC_WORKSPACE_BYTES];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_address[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device, resolved once per device.
+int scratch_on_current_device(void** address, const char* who) {
+    int device = -1;
+    AEON_HIP(hipGetDevice(&device));
+    AEON_REQUIRE(device >= 0 && device < kMaxDevices, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: device ordinal %d is outside the %d this entry point keeps an address for",
+                 who, device, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_address[device] == nullptr) {
+        void* resolved = nullptr;
+        AEON_HIP(hipGetSymbolAddress(&resolved, HIP_SYMBOL(scratch)));
+        AEON_REQUIRE(resolved != nullptr, AEON_ERR_HIP, "%s: the scratch array has no address on device %d",
+                     who, device);
+        g_scratch_address[device] = resolved;
+    }
+    *address = g_scratch_address[device];
+    return AEON_OK;
+}
+
+}  // namespace
+
+extern "C" int aeon_moe_layer_decode_noalloc(const aeon_moe_layer* layer, const void* d_x,
+                                             int x_stride, int tokens, void* d_out, int out_stride,
+                                             int32_t* d_topk_ids, float* d_topk_weights,
+                                             void* stream) {
+    const char* who = "aeon_moe_layer_decode_noalloc";
+    if (int rc = check_layer(layer, who)) return rc;
+    AEON_REQUIRE(tokens >= 0, AEON_ERR_INVALID_ARGUMENT, "%s: bad token count %d", who, tokens);
+    if (tokens == 0) return AEON_OK;
+    AEON_REQUIRE(positions_fit(*layer, tokens), AEON_ERR_INVALID_ARGUMENT,
+                 "%s: %d tokens x top-%d exceed 32-bit positions", who, tokens, layer->top_k);
+    const size_t needed = carve(*layer, tokens, nullptr).bytes;
+    AEON_REQUIRE(needed <= sizeof(scratch), AEON_ERR_INVALID_ARGUMENT,
+                 "%s: %d tokens at hidden %d / intermediate %d / top-%d of %d experts need a workspace "
+                 "of %zu bytes; the built-in one holds %zu (use aeon_moe_layer_decode with a workspace "
+                 "of the caller's)", who, tokens, layer->hidden, layer->intermediate, layer->top_k,
+                 layer->experts, needed, sizeof(scratch));
+    void* workspace = nullptr;
+    if (int rc = scratch_on_current_device(&workspace, who)) return rc;
+    return aeon_moe_layer_decode(layer, d_x, x_stride, tokens, d_out, out_stride, d_topk_ids,
+                                 d_topk_weights, workspace, sizeof(scratch), stream);
 }
 
 extern "C" const float* aeon_moe_layer_logits(const aeon_moe_layer* layer, int tokens,
