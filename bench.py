@@ -365,7 +365,8 @@ def run_other_configs(pool, layer, moe, capi, synth, torch, np, H, I, E, K_TOP, 
     def gemv(i):
         s = i % pool.slots
         capi.call("aeon_a64_gemv", capi.vp(x1), H, C.c_void_p(int(tab[s, 0])),
-                  C.c_void_p(int(tab[s, 1])), capi.vp(y1), I, 1, I, H, moe.stream_ptr())
+                  C.c_void_p(int(tab[s, 1])), pool.scale_group, capi.vp(y1), I, 1, I, H,
+                  moe.stream_ptr())
 
     ms = timed(gemv, reps)
     b0 = bm + H * 2 + I * 2
@@ -384,7 +385,7 @@ def run_other_configs(pool, layer, moe, capi, synth, torch, np, H, I, E, K_TOP, 
 
         def expert(i):
             capi.call("aeon_a64_expert_decode", capi.vp(x), tokens, C.byref(structs[i % pool.slots]),
-                      capi.vp(w), capi.vp(hidden), capi.vp(contrib), None, capi.vp(out), H, I,
+                      pool.scale_group, capi.vp(w), capi.vp(hidden), capi.vp(contrib), None, capi.vp(out), H, I,
                       C.c_float(LIMIT), 1, moe.stream_ptr())
 
         ms = timed(expert, reps)
@@ -656,7 +657,7 @@ def main():
                 p = torch.empty(n * k // 2, dtype=torch.uint8, device="cuda")
                 sc = torch.empty(n * k // 32, dtype=torch.int16, device="cuda")
                 capi.call("aeon_synth_matrix_swizzled", C.c_uint64(SEED), expert, m, n, k, cfg[0],
-                          cfg[1], capi.vp(p), capi.vp(sc), moe.stream_ptr())
+                          cfg[1], 128, capi.vp(p), capi.vp(sc), moe.stream_ptr())
                 mats.append((p.cpu().numpy().view(np.uint32), sc.cpu().numpy().view(np.uint16)))
             return mats
 

@@ -53,21 +53,29 @@ int aeon_unswizzle_w4a16(const uint32_t* src_packed, const uint16_t* src_scale,
  * (src/backend/swizzled_w4a16/core/swizzled_expert_format.hpp:9-30 is the layout it reads).
  * A tile is 16 rows x 128 columns = 64 lanes x 16 bytes, tiles ordered [row/16][column/128];
  * lane l holds row l%16 and, in word s of its uint4, columns 128g+32s+8(l/16)+0..7 in the
- * payload's own nibble order; one fp16 scale per (row, 128-column group) at [tile][row%16].
- * Requires N%16==0, K%128==0. Sizes in bytes: */
+ * payload's own nibble order. Requires N%16==0, K%128==0.
+ * `scale_group` (everywhere below) is the number of columns one fp16 scale covers:
+ *   32  -- the payload's own scales, all kept (swizzled_expert_format.hpp:18-23: one per 32
+ *          columns): [tile][row%16][s], s = 0..3 the scale of columns 128g+32s..+31;
+ *   128 -- one scale per (row, 128 columns) at [tile][row%16], a quarter of the scale bytes;
+ *          only for payloads whose four group-32 scales inside every 128 columns are bit-equal.
+ * Sizes in bytes (aeon_a64_scale_bytes is 0 for any other scale_group): */
 size_t aeon_a64_packed_bytes(int N, int K);
-size_t aeon_a64_scale_bytes(int N, int K);
-/* Host repack of one swizzled matrix. Fails with AEON_ERR_INVALID_ARGUMENT when the four
- * group-32 scales of any 128-group are not bit-equal (the layout stores one). */
+size_t aeon_a64_scale_bytes(int N, int K, int scale_group);
+/* Host repack of one swizzled matrix. With scale_group 128 it fails with
+ * AEON_ERR_INVALID_ARGUMENT when the four group-32 scales of any 128 columns are not bit-equal. */
 int aeon_a64_repack_host(const uint32_t* swz_packed, const uint16_t* swz_scale, int N, int K,
-                         int rpw, int lpr, uint32_t* a64_packed, uint16_t* a64_scale);
+                         int rpw, int lpr, int scale_group, uint32_t* a64_packed,
+                         uint16_t* a64_scale);
 int aeon_a64_unrepack_host(const uint32_t* a64_packed, const uint16_t* a64_scale, int N, int K,
-                           int rpw, int lpr, uint32_t* swz_packed, uint16_t* swz_scale);
-/* Device repack (one launch). `d_mismatch` (int, nullable) is incremented once per 128-group
- * whose four group-32 scales differ; the caller zeroes and reads it. */
+                           int rpw, int lpr, int scale_group, uint32_t* swz_packed,
+                           uint16_t* swz_scale);
+/* Device repack (one launch). With scale_group 128, `d_mismatch` (int, nullable) is incremented
+ * once per 128 columns of a row whose four group-32 scales differ; the caller zeroes and reads
+ * it, and a non-zero count means the result must not be used. */
 int aeon_a64_repack_device(const void* d_swz_packed, const void* d_swz_scale, int N, int K,
-                           int rpw, int lpr, void* d_a64_packed, void* d_a64_scale,
-                           int* d_mismatch, void* stream);
+                           int rpw, int lpr, int scale_group, void* d_a64_packed,
+                           void* d_a64_scale, int* d_mismatch, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Decode kernels over the `.aeon` swizzled layout (the drop-in entry points)
@@ -164,19 +172,20 @@ int aeon_moe_grouped_w2(const void* d_expert_hidden, const int* d_expert_offsets
  * ---------------------------------------------------------------------------------------- */
 
 /* W4A16 GEMV over an A64 matrix: same arithmetic contract as
- * dispatch_aeon_w4a16_swizzled_gemv (aeon_w4a16_swizzled_gemv.hpp:43-93,166-190) with one
- * scale per 128 columns. VALU only (no MFMA): 1 KiB coalesced wave loads, in-register nibble
+ * dispatch_aeon_w4a16_swizzled_gemv (aeon_w4a16_swizzled_gemv.hpp:43-93,166-190): the scale is
+ * applied in fp32 to the dot product of each scale group. VALU only (no MFMA): 1 KiB coalesced wave loads, in-register nibble
  * dequant, K split across the waves of a workgroup and reduced by wave shuffles.
  * `tokens` activations [tokens][K] (row pitch x_stride elements) give [tokens][N] outputs
  * (pitch out_stride); 1 <= tokens <= 8. */
 int aeon_a64_gemv(const void* d_x, int x_stride, const void* d_packed, const void* d_scale,
-                  void* d_out, int out_stride, int tokens, int N, int K, void* stream);
+                  int scale_group, void* d_out, int out_stride, int tokens, int N, int K,
+                  void* stream);
 /* dispatch_aeon_w4a16_swizzled_dual_gemv (aeon_w4a16_swizzled_gemv.hpp:95-164,192-222) on A64:
  * two matrices, one activation read. */
 int aeon_a64_dual_gemv(const void* d_x, int x_stride, const void* d_packed_a,
                        const void* d_scale_a, const void* d_packed_b, const void* d_scale_b,
-                       void* d_out_a, void* d_out_b, int out_stride, int tokens, int N, int K,
-                       void* stream);
+                       int scale_group, void* d_out_a, void* d_out_b, int out_stride, int tokens,
+                       int N, int K, void* stream);
 
 /* One expert's six A64 sub-tensors (device pointers): the wave64 counterpart of the slot
  * views UnifiedVRAMExpertPool::get_w{1,2,3}_{packed,scale} return
@@ -198,7 +207,7 @@ typedef struct {
  * slot: out[t] = half(float(shared[t]) + contrib[t]); d_shared nullable, may alias d_out.
  * use_mfma 0 = VALU GEMV kernels (tokens <= 8), 1 = the MFMA segment kernels. */
 int aeon_a64_expert_decode(const void* d_x, int tokens, const aeon_a64_expert* expert,
-                           const float* d_route_weights, void* d_hidden, float* d_contrib,
+                           int scale_group, const float* d_route_weights, void* d_hidden, float* d_contrib,
                            const void* d_shared, void* d_out, int H, int I, float swiglu_limit,
                            int use_mfma, void* stream);
 
@@ -256,6 +265,7 @@ typedef struct {
     const float* d_router_weight; /* fp32 [hidden][experts]; only aeon_moe_layer_decode reads it */
     const float* d_router_bias;   /* fp32 [experts], nullable */
     const aeon_a64_expert* d_experts;
+    int scale_group; /* columns per scale of every expert in the table: 128 (0 reads as 128) or 32 */
 } aeon_moe_layer;
 
 size_t aeon_moe_layer_workspace_bytes(const aeon_moe_layer* layer, int max_tokens);
@@ -402,30 +412,35 @@ int aeon_payload_layout_for(int hidden, int intermediate, aeon_payload_layout* o
  * six device views of the slot at `d_slot` -- the counterpart of UnifiedVRAMExpertPool's slot
  * views (src/backend/swizzled_w4a16/core/vram_expert_pool.hpp:22-82) with every expert
  * resident. */
-size_t aeon_a64_slot_bytes(int hidden, int intermediate);
-int aeon_a64_slot_views(void* d_slot, int hidden, int intermediate, aeon_a64_expert* out);
+size_t aeon_a64_slot_bytes(int hidden, int intermediate, int scale_group);
+int aeon_a64_slot_views(void* d_slot, int hidden, int intermediate, int scale_group,
+                        aeon_a64_expert* out);
 
 /* Loads experts [first, first+count) of `layer` into consecutive slots of `d_pool` (slot i at
  * d_pool + i*aeon_a64_slot_bytes): payload bytes are copied from the mapping to a device staging
  * buffer and re-swizzled there into the wave64 packing, copy and repack of neighbouring experts
  * overlapped on two streams of the library's own. `h_table[i]` receives
  * the views of slot i (host array; copy it to the device as the layer's expert table).
- * Blocks until the pool is complete. `*mismatches` (nullable) = number of 128-column groups
- * whose four group-32 scales were not bit-equal (the wave64 packing stores one; must be 0). */
+ * Blocks until the pool is complete. scale_group 32 keeps every scale of the container (the
+ * choice for a real checkpoint); with 128 a payload whose four group-32 scales differ anywhere
+ * inside 128 columns makes the call fail with AEON_ERR_INVALID_ARGUMENT (the pool is then not to
+ * be used), never a pool that computes with the wrong weights. */
 int aeon_resident_load_layer(const aeon_expert_catalog* catalog, uint32_t layer, uint32_t first,
-                             uint32_t count, int hidden, int intermediate, void* d_pool,
-                             size_t pool_bytes, aeon_a64_expert* h_table, long* mismatches);
+                             uint32_t count, int hidden, int intermediate, int scale_group,
+                             void* d_pool, size_t pool_bytes, aeon_a64_expert* h_table);
 
 /* ------------------------------------------------------------------------------------------
  * Synthetic experts on the device (benchmarks and tests)
  * ---------------------------------------------------------------------------------------- */
 
 /* Fills one matrix (matrix 0 = W1, 1 = W3, 2 = W2) of synthetic expert `expert` directly in
- * device memory in the `.aeon` swizzled layout (packed N*K/2 bytes, scales N*K/32 fp16 with
- * each group-128 scale replicated over its four group-32 slots): int4 uniform in [-8,7],
- * scales uniform in [0.005,0.02], a pure function of (seed, expert, matrix, index). */
+ * device memory in the `.aeon` swizzled layout (packed N*K/2 bytes, scales N*K/32 fp16): int4
+ * uniform in [-8,7], scales uniform in [0.005,0.02] -- with scale_group 128 one per (row, 128
+ * columns) replicated over its four group-32 slots, with 32 one of its own per slot -- a pure
+ * function of (seed, expert, matrix, index). */
 int aeon_synth_matrix_swizzled(uint64_t seed, int expert, int matrix, int N, int K, int rpw,
-                               int lpr, void* d_packed, void* d_scale, void* stream);
+                               int lpr, int scale_group, void* d_packed, void* d_scale,
+                               void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Measurement aid (no counterpart in the reference)

@@ -565,6 +565,12 @@ void orc_hc_post(const double* layer_out, const double* residual, const double* 
 /* ------------------------------------------------------------------------------------ */
 
 orc_a64_addr orc_a64_address(int columns, int row, int column) {
+    return orc_a64_address_g(columns, row, column, 128);
+}
+
+/* scale_group 128: one scale per (row, 128 columns) at [tile][row%16]; 32: the row's four
+ * group-32 scales of the 128 columns side by side, [tile][row%16][step]. */
+orc_a64_addr orc_a64_address_g(int columns, int row, int column, int scale_group) {
     const int groups = columns / 128;
     const int tile_row = row / 16;
     const int r = row % 16;
@@ -577,22 +583,33 @@ orc_a64_addr orc_a64_address(int columns, int row, int column) {
     orc_a64_addr a;
     a.packed_word = (tile * 64u + (size_t)lane) * 4u + (size_t)s;
     a.nibble = nibble_slot(column % 8);
-    a.scale_index = tile * 16u + (size_t)r;
+    a.scale_index = scale_group == 32 ? (tile * 16u + (size_t)r) * 4u + (size_t)s
+                                      : tile * 16u + (size_t)r;
     return a;
 }
 
 int orc_a64_pack(const uint32_t* src_packed, const uint16_t* src_scale32,
                  int rows, int columns, uint32_t* a64_packed, uint16_t* a64_scale) {
+    return orc_a64_pack_g(src_packed, src_scale32, rows, columns, 128, a64_packed, a64_scale);
+}
+
+int orc_a64_pack_g(const uint32_t* src_packed, const uint16_t* src_scale32, int rows, int columns,
+                   int scale_group, uint32_t* a64_packed, uint16_t* a64_scale) {
     if (rows <= 0 || columns <= 0 || rows % 16 != 0 || columns % 128 != 0) return -1;
+    if (scale_group != 128 && scale_group != 32) return -3;
     const int groups32 = columns / 32;
     memset(a64_packed, 0, (size_t)rows * (size_t)columns / 2);
     for (int row = 0; row < rows; ++row) {
         for (int column = 0; column < columns; ++column) {
             const uint32_t word = src_packed[(size_t)row * (columns / 8) + column / 8];
             const uint32_t q = (word >> (4 * (column % 8))) & 0xFu;
-            const orc_a64_addr a = orc_a64_address(columns, row, column);
+            const orc_a64_addr a = orc_a64_address_g(columns, row, column, scale_group);
             a64_packed[a.packed_word] |= q << (4 * a.nibble);
-            if (column % 128 == 0) {
+            if (scale_group == 32) {
+                if (column % 32 == 0) {
+                    a64_scale[a.scale_index] = src_scale32[(size_t)row * groups32 + column / 32];
+                }
+            } else if (column % 128 == 0) {
                 const uint16_t* s = src_scale32 + (size_t)row * groups32 + column / 32;
                 if (s[0] != s[1] || s[0] != s[2] || s[0] != s[3]) return -2;
                 a64_scale[a.scale_index] = s[0];
@@ -604,9 +621,14 @@ int orc_a64_pack(const uint32_t* src_packed, const uint16_t* src_scale32,
 
 void orc_a64_decode(const uint32_t* a64_packed, const uint16_t* a64_scale,
                     int rows, int columns, double* out) {
+    orc_a64_decode_g(a64_packed, a64_scale, rows, columns, 128, out);
+}
+
+void orc_a64_decode_g(const uint32_t* a64_packed, const uint16_t* a64_scale, int rows, int columns,
+                      int scale_group, double* out) {
     for (int row = 0; row < rows; ++row)
         for (int column = 0; column < columns; ++column) {
-            const orc_a64_addr a = orc_a64_address(columns, row, column);
+            const orc_a64_addr a = orc_a64_address_g(columns, row, column, scale_group);
             const int q = (int)((a64_packed[a.packed_word] >> (4 * a.nibble)) & 0xFu);
             out[(size_t)row * columns + column] =
                 (double)(q - 8) * orc_half_bits_to_double(a64_scale[a.scale_index]);

@@ -150,6 +150,13 @@ void orc_hc_post(const double* layer_out, const double* residual, const double* 
  * Addresses are written out scalar by scalar, as orc_swizzled_address is. */
 typedef struct { size_t packed_word; int nibble; size_t scale_index; } orc_a64_addr;
 orc_a64_addr orc_a64_address(int columns, int row, int column);
+/* The same with the scale grouping stated: 128 (as above) or 32 (four scales kept per 128
+ * columns, [tile][row%16][32-column step]). */
+orc_a64_addr orc_a64_address_g(int columns, int row, int column, int scale_group);
+int orc_a64_pack_g(const uint32_t* src_packed, const uint16_t* src_scale32, int rows, int columns,
+                   int scale_group, uint32_t* a64_packed, uint16_t* a64_scale);
+void orc_a64_decode_g(const uint32_t* a64_packed, const uint16_t* a64_scale, int rows, int columns,
+                      int scale_group, double* out);
 /* From the source layout. Returns -1 on a bad shape (rows%16, columns%128) and -2 when the
  * four group-32 scales of a 128-group are not bit-equal. */
 int orc_a64_pack(const uint32_t* src_packed, const uint16_t* src_scale32,

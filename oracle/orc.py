@@ -149,10 +149,10 @@ def swizzled_address(columns, rpw, lpr, row, column):
     return a.storage_slot, a.packed_word, a.nibble
 
 
-def a64_address(columns, row, column):
-    f = lib().orc_a64_address
+def a64_address(columns, row, column, scale_group=128):
+    f = lib().orc_a64_address_g
     f.restype = _A64Addr
-    a = f(columns, row, column)
+    a = f(columns, row, column, scale_group)
     return a.packed_word, a.nibble, a.scale_index
 
 
@@ -174,24 +174,24 @@ def swizzled_encode(w, rows, columns, rpw, lpr):
     return p, s
 
 
-def a64_pack(src_packed, src_scale32, rows, columns):
+def a64_pack(src_packed, src_scale32, rows, columns, scale_group=128):
     sp = np.ascontiguousarray(src_packed, dtype=np.uint32)
     ss = np.ascontiguousarray(src_scale32).view(np.uint16)
     p = np.empty(rows * columns // 8, dtype=np.uint32)
-    s = np.empty(rows * columns // 128, dtype=np.uint16)
-    rc = lib().orc_a64_pack(_ptr(sp, C.c_uint32), _ptr(ss, C.c_uint16), rows, columns,
-                            _ptr(p, C.c_uint32), _ptr(s, C.c_uint16))
+    s = np.empty(rows * columns // scale_group, dtype=np.uint16)
+    rc = lib().orc_a64_pack_g(_ptr(sp, C.c_uint32), _ptr(ss, C.c_uint16), rows, columns,
+                              scale_group, _ptr(p, C.c_uint32), _ptr(s, C.c_uint16))
     if rc != 0:
         raise ValueError("orc_a64_pack failed with %d" % rc)
     return p, s
 
 
-def a64_decode(a64_packed, a64_scale, rows, columns):
+def a64_decode(a64_packed, a64_scale, rows, columns, scale_group=128):
     p = np.ascontiguousarray(a64_packed, dtype=np.uint32)
     s = np.ascontiguousarray(a64_scale).view(np.uint16)
     out = np.empty((rows, columns), dtype=np.float64)
-    lib().orc_a64_decode(_ptr(p, C.c_uint32), _ptr(s, C.c_uint16), rows, columns,
-                         _ptr(out, C.c_double))
+    lib().orc_a64_decode_g(_ptr(p, C.c_uint32), _ptr(s, C.c_uint16), rows, columns, scale_group,
+                           _ptr(out, C.c_double))
     return out
 
 

@@ -72,11 +72,11 @@ struct SlotLayout {
     size_t bytes;
 };
 
-SlotLayout slot_layout(int hidden, int intermediate) {
+SlotLayout slot_layout(int hidden, int intermediate, int scale_group) {
     const size_t sizes[6] = {
-        aeon_a64_packed_bytes(intermediate, hidden), aeon_a64_scale_bytes(intermediate, hidden),
-        aeon_a64_packed_bytes(intermediate, hidden), aeon_a64_scale_bytes(intermediate, hidden),
-        aeon_a64_packed_bytes(hidden, intermediate), aeon_a64_scale_bytes(hidden, intermediate)};
+        aeon_a64_packed_bytes(intermediate, hidden), aeon_a64_scale_bytes(intermediate, hidden, scale_group),
+        aeon_a64_packed_bytes(intermediate, hidden), aeon_a64_scale_bytes(intermediate, hidden, scale_group),
+        aeon_a64_packed_bytes(hidden, intermediate), aeon_a64_scale_bytes(hidden, intermediate, scale_group)};
     SlotLayout l{};
     size_t at = 0;
     for (int i = 0; i < 6; ++i) {
@@ -218,17 +218,21 @@ extern "C" int aeon_payload_layout_for(int hidden, int intermediate, aeon_payloa
     return AEON_OK;
 }
 
-extern "C" size_t aeon_a64_slot_bytes(int hidden, int intermediate) {
+extern "C" size_t aeon_a64_slot_bytes(int hidden, int intermediate, int scale_group) {
     if (hidden <= 0 || intermediate <= 0 || hidden % 128 != 0 || intermediate % 128 != 0) return 0;
-    return slot_layout(hidden, intermediate).bytes;
+    if (scale_group != 128 && scale_group != 32) return 0;
+    return slot_layout(hidden, intermediate, scale_group).bytes;
 }
 
-extern "C" int aeon_a64_slot_views(void* d_slot, int hidden, int intermediate, aeon_a64_expert* out) {
+extern "C" int aeon_a64_slot_views(void* d_slot, int hidden, int intermediate, int scale_group,
+                                   aeon_a64_expert* out) {
     AEON_REQUIRE(d_slot != nullptr && out != nullptr, AEON_ERR_INVALID_ARGUMENT, "aeon_a64_slot_views: null argument");
     AEON_REQUIRE(hidden > 0 && intermediate > 0 && hidden % 128 == 0 && intermediate % 128 == 0,
                  AEON_ERR_INVALID_ARGUMENT, "aeon_a64_slot_views: the wave64 packing needs multiples of 128 "
                  "(hidden=%d intermediate=%d)", hidden, intermediate);
-    const SlotLayout l = slot_layout(hidden, intermediate);
+    AEON_REQUIRE(scale_group == 128 || scale_group == 32, AEON_ERR_INVALID_ARGUMENT,
+                 "aeon_a64_slot_views: scale_group must be 128 or 32, not %d", scale_group);
+    const SlotLayout l = slot_layout(hidden, intermediate, scale_group);
     char* base = static_cast<char*>(d_slot);
     out->w1_packed = base + l.offset[0];
     out->w1_scale = base + l.offset[1];
@@ -261,12 +265,14 @@ struct LoadResources {
 
 extern "C" int aeon_resident_load_layer(const aeon_expert_catalog* catalog, uint32_t layer,
                                         uint32_t first, uint32_t count, int hidden,
-                                        int intermediate, void* d_pool, size_t pool_bytes,
-                                        aeon_a64_expert* h_table, long* mismatches) {
+                                        int intermediate, int scale_group, void* d_pool,
+                                        size_t pool_bytes, aeon_a64_expert* h_table) {
     const char* who = "aeon_resident_load_layer";
     AEON_REQUIRE(catalog != nullptr && d_pool != nullptr && h_table != nullptr, AEON_ERR_INVALID_ARGUMENT,
                  "%s: null argument", who);
     if (int rc = check_expert_shape(hidden, intermediate, who)) return rc;
+    AEON_REQUIRE(scale_group == 128 || scale_group == 32, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: scale_group must be 128 or 32, not %d", who, scale_group);
     AEON_REQUIRE(layer < catalog->layers && first <= catalog->experts_per_layer &&
                      count <= catalog->experts_per_layer - first,
                  AEON_ERR_OUT_OF_RANGE, "%s: experts [%u, %u) of layer %u are outside the %u x %u catalog",
@@ -277,10 +283,9 @@ extern "C" int aeon_resident_load_layer(const aeon_expert_catalog* catalog, uint
                  "%s: an expert of shape (%d, %d) is %zu bytes in the container's layout, the catalog's "
                  "payloads are %llu", who, hidden, intermediate, payload.total,
                  static_cast<unsigned long long>(catalog->payload_bytes));
-    const SlotLayout slot = slot_layout(hidden, intermediate);
+    const SlotLayout slot = slot_layout(hidden, intermediate, scale_group);
     AEON_REQUIRE(pool_bytes >= static_cast<size_t>(count) * slot.bytes, AEON_ERR_INVALID_ARGUMENT,
                  "%s: pool of %zu bytes cannot hold %u slots of %zu", who, pool_bytes, count, slot.bytes);
-    if (mismatches) *mismatches = 0;
     if (count == 0) return AEON_OK;
 
     LoadResources r;
@@ -305,7 +310,7 @@ extern "C" int aeon_resident_load_layer(const aeon_expert_catalog* catalog, uint
         AEON_HIP(hipMemcpyAsync(r.staged[b], catalog->base + catalog->offsets[entry], payload.total,
                                 hipMemcpyHostToDevice, r.stream[b]));
         char* d_slot = static_cast<char*>(d_pool) + static_cast<size_t>(i) * slot.bytes;
-        if (int rc = aeon_a64_slot_views(d_slot, hidden, intermediate, &h_table[i])) return rc;
+        if (int rc = aeon_a64_slot_views(d_slot, hidden, intermediate, scale_group, &h_table[i])) return rc;
         void* dst_packed[3] = {const_cast<void*>(h_table[i].w1_packed), const_cast<void*>(h_table[i].w3_packed),
                                const_cast<void*>(h_table[i].w2_packed)};
         void* dst_scale[3] = {const_cast<void*>(h_table[i].w1_scale), const_cast<void*>(h_table[i].w3_scale),
@@ -315,8 +320,8 @@ extern "C" int aeon_resident_load_layer(const aeon_expert_catalog* catalog, uint
             const bool down = m == 2;  // W2 is [hidden][intermediate] with the (8, 4) swizzle
             if (int rc = aeon_a64_repack_device(src + sub_offset[m], src + sub_scale[m],
                                                 down ? hidden : intermediate, down ? intermediate : hidden,
-                                                down ? 8 : 4, down ? 4 : 8, dst_packed[m], dst_scale[m],
-                                                r.d_mismatch, r.stream[b])) {
+                                                down ? 8 : 4, down ? 4 : 8, scale_group, dst_packed[m],
+                                                dst_scale[m], r.d_mismatch, r.stream[b])) {
                 return rc;
             }
         }
@@ -326,6 +331,11 @@ extern "C" int aeon_resident_load_layer(const aeon_expert_catalog* catalog, uint
     AEON_HIP(hipStreamSynchronize(r.stream[1]));
     int found = 0;
     AEON_HIP(hipMemcpy(&found, r.d_mismatch, sizeof(int), hipMemcpyDeviceToHost));
-    if (mismatches) *mismatches = found;
+    // One scale per 128 columns only holds a payload whose four group-32 scales agree there: a
+    // pool built from any other payload would compute with wrong weights, so it is an error, and
+    // the pool's contents are not to be used.
+    AEON_REQUIRE(found == 0, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: %d 128-column groups of layer %u carry four different group-32 scales; load with "
+                 "scale_group 32 to keep them", who, found, layer);
     return AEON_OK;
 }

@@ -1,7 +1,8 @@
 // Decode kernels over the wave64 ("A64") packing.
 //
 // Two families, both HBM-bound by construction (every weight byte is read once per segment in
-// 1 KiB coalesced wave loads, scales at one fp16 per 128 columns):
+// 1 KiB coalesced wave loads; scales at one fp16 per 128 columns, or -- template parameter
+// SG = 4 -- the payload's own four per 128 columns, one per 32-column MFMA step):
 //
 //   * a64_gemv_kernel: VALU only. Lane (row l%16, chunk l/16) dequantises its 32 nibbles in
 //     registers and feeds v_dot2_f32_f16 against four 16-byte activation chunks; the four
@@ -41,9 +42,10 @@ struct GemvArgs {
     float limit;
     const float* tok_weight;
     float* out_f32;
+    int scales_per_group;  // 1 (one fp16 per row and 128 columns) or 4 (one per 32 columns)
 };
 
-template <int NMAT, int TOK, int WK>
+template <int NMAT, int TOK, int WK, int SG>
 __global__ __launch_bounds__(WK * 64) void a64_gemv_kernel(GemvArgs a) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -60,16 +62,21 @@ __global__ __launch_bounds__(WK * 64) void a64_gemv_kernel(GemvArgs a) {
 
     for (int g0 = wave; g0 < a.groups; g0 += WK * kGemvPrefetch) {
         uint4 wq[NMAT][kGemvPrefetch];
-        uint16_t sc[NMAT][kGemvPrefetch];
+        // the row's scale(s) of the group: one fp16, or four (MFMA-step order) in 8 bytes
+        uint2 sc[NMAT][kGemvPrefetch];
+        auto load_scale = [&](const uint16_t* base, int g) {
+            if (SG == 4) return *reinterpret_cast<const uint2*>(base + ((tile_base + g) * 16 + r) * 4);
+            return make_uint2(base[(tile_base + g) * 16 + r], 0u);
+        };
 #pragma unroll
         for (int j = 0; j < kGemvPrefetch; ++j) {
             const int g = g0 + j * WK;
             if (g < a.groups) {
                 wq[0][j] = a.pa[(tile_base + g) * 64 + lane];
-                sc[0][j] = a.sa[(tile_base + g) * 16 + r];
+                sc[0][j] = load_scale(a.sa, g);
                 if (NMAT == 2) {
                     wq[1][j] = a.pb[(tile_base + g) * 64 + lane];
-                    sc[1][j] = a.sb[(tile_base + g) * 16 + r];
+                    sc[1][j] = load_scale(a.sb, g);
                 }
             }
         }
@@ -87,12 +94,25 @@ __global__ __launch_bounds__(WK * 64) void a64_gemv_kernel(GemvArgs a) {
                         const uint4 x3 = *reinterpret_cast<const uint4*>(xp + 96);
 #pragma unroll
                         for (int m = 0; m < NMAT; ++m) {
-                            float d = 0.0f;
-                            d = dot8(wq[m][j].x, x0, d);
-                            d = dot8(wq[m][j].y, x1, d);
-                            d = dot8(wq[m][j].z, x2, d);
-                            d = dot8(wq[m][j].w, x3, d);
-                            acc[m][t] += half_bits_to_float(sc[m][j]) * d;
+                            if (SG == 4) {
+                                // word s of the lane holds columns of 32-column group s only
+                                const uint2 s4 = sc[m][j];
+                                acc[m][t] += half_bits_to_float(static_cast<uint16_t>(s4.x & 0xFFFFu)) *
+                                             dot8(wq[m][j].x, x0, 0.0f);
+                                acc[m][t] += half_bits_to_float(static_cast<uint16_t>(s4.x >> 16)) *
+                                             dot8(wq[m][j].y, x1, 0.0f);
+                                acc[m][t] += half_bits_to_float(static_cast<uint16_t>(s4.y & 0xFFFFu)) *
+                                             dot8(wq[m][j].z, x2, 0.0f);
+                                acc[m][t] += half_bits_to_float(static_cast<uint16_t>(s4.y >> 16)) *
+                                             dot8(wq[m][j].w, x3, 0.0f);
+                            } else {
+                                float d = 0.0f;
+                                d = dot8(wq[m][j].x, x0, d);
+                                d = dot8(wq[m][j].y, x1, d);
+                                d = dot8(wq[m][j].z, x2, d);
+                                d = dot8(wq[m][j].w, x3, d);
+                                acc[m][t] += half_bits_to_float(static_cast<uint16_t>(sc[m][j].x)) * d;
+                            }
                         }
                     }
                 }
@@ -136,18 +156,24 @@ __global__ __launch_bounds__(WK * 64) void a64_gemv_kernel(GemvArgs a) {
     }
 }
 
-template <int NMAT, int TOK>
-static int launch_gemv_wk(const GemvArgs& a, int wk, hipStream_t stream) {
+template <int NMAT, int TOK, int SG>
+static int launch_gemv_wk_sg(const GemvArgs& a, int wk, hipStream_t stream) {
     const dim3 grid(a.N / 16);
     if (wk >= 16) {
-        a64_gemv_kernel<NMAT, TOK, 16><<<grid, 16 * 64, 0, stream>>>(a);
+        a64_gemv_kernel<NMAT, TOK, 16, SG><<<grid, 16 * 64, 0, stream>>>(a);
     } else if (wk >= 8) {
-        a64_gemv_kernel<NMAT, TOK, 8><<<grid, 8 * 64, 0, stream>>>(a);
+        a64_gemv_kernel<NMAT, TOK, 8, SG><<<grid, 8 * 64, 0, stream>>>(a);
     } else {
-        a64_gemv_kernel<NMAT, TOK, 4><<<grid, 4 * 64, 0, stream>>>(a);
+        a64_gemv_kernel<NMAT, TOK, 4, SG><<<grid, 4 * 64, 0, stream>>>(a);
     }
     AEON_LAUNCH_CHECK();
     return AEON_OK;
+}
+
+template <int NMAT, int TOK>
+static int launch_gemv_wk(const GemvArgs& a, int wk, hipStream_t stream) {
+    return a.scales_per_group == 4 ? launch_gemv_wk_sg<NMAT, TOK, 4>(a, wk, stream)
+                                   : launch_gemv_wk_sg<NMAT, TOK, 1>(a, wk, stream);
 }
 
 template <int NMAT>
@@ -162,9 +188,11 @@ static int launch_gemv(const GemvArgs& a, hipStream_t stream) {
     return launch_gemv_wk<NMAT, 8>(a, wk > 8 ? 8 : wk, stream);
 }
 
-static int check_a64_shape(int N, int K, const char* who) {
+static int check_a64_shape(int N, int K, int scale_group, const char* who) {
     AEON_REQUIRE(N > 0 && K > 0 && N % 16 == 0 && K % 128 == 0, AEON_ERR_INVALID_ARGUMENT,
                  "%s: the wave64 packing needs N%%16==0 and K%%128==0 (N=%d K=%d)", who, N, K);
+    AEON_REQUIRE(scale_group == 128 || scale_group == 32, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: scale_group must be 128 or 32, not %d", who, scale_group);
     return AEON_OK;
 }
 
@@ -172,27 +200,97 @@ static int check_a64_shape(int N, int K, const char* who) {
 // MFMA segment kernels
 // ---------------------------------------------------------------------------------------------
 
-__device__ __forceinline__ float4_t mfma_group(const u32x4_t& wq, const half8_t xf[4]) {
-    float4_t t = {0.0f, 0.0f, 0.0f, 0.0f};
-    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(unpack8_vec(wq[0]), xf[0], t, 0, 0, 0);
-    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(unpack8_vec(wq[1]), xf[1], t, 0, 0, 0);
-    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(unpack8_vec(wq[2]), xf[2], t, 0, 0, 0);
-    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(unpack8_vec(wq[3]), xf[3], t, 0, 0, 0);
-    return t;
+// The matrix instruction is issued with the token rows as its first operand and the weight tile
+// as its second: lane l supplies token l%16 / weight row l%16 and the 8-column chunk l/16 of a
+// 32-column step (the two operands have the same lane pattern, so the packed tile needs no
+// movement either way round) and ends up holding tokens 4*(l/16)..+3 of weight row l%16. A lane
+// therefore needs the scales of one weight row only: one fp16 per 128 columns, or the row's four
+// (one per 32-column step, 8 bytes side by side).
+template <int SG>
+struct RowScales;
+template <>
+struct RowScales<1> {
+    uint16_t v;
+    // `tile_scales` = the 16 rows' scales of one (tile, 128-column group), in memory or in LDS
+    __device__ __forceinline__ void load(const AEON_GLOBAL uint16_t* tile_scales, int row) { v = tile_scales[row]; }
+    __device__ __forceinline__ void load_lds(const uint16_t* tile_scales, int row) { v = tile_scales[row]; }
+    __device__ __forceinline__ float get(int) const { return half_bits_to_float(v); }
+};
+template <>
+struct RowScales<4> {
+    u32x2_t v;
+    __device__ __forceinline__ void load(const AEON_GLOBAL uint16_t* tile_scales, int row) {
+        v = *reinterpret_cast<const AEON_GLOBAL u32x2_t*>(tile_scales + row * 4);
+    }
+    __device__ __forceinline__ void load_lds(const uint16_t* tile_scales, int row) {
+        v = *reinterpret_cast<const u32x2_t*>(tile_scales + row * 4);
+    }
+    __device__ __forceinline__ float get(int st) const {
+        const uint32_t w = v[st >> 1];
+        return half_bits_to_float(static_cast<uint16_t>((st & 1) ? (w >> 16) : (w & 0xFFFFu)));
+    }
+};
+
+// acc (tokens 4*(l/16)..+3 of weight row l%16) += the scaled product of one weight tile with the
+// 16 token rows over one 128-column group. One scale per row: the four steps chain into one
+// result, scaled once. Four per row: every step is a product of its own, scaled by the step's
+// scale. In fp32 either way, so the dequantisation stays exact.
+template <int SG>
+__device__ __forceinline__ void mfma_scaled(float4_t& acc, const u32x4_t& wq, const half8_t xf[4],
+                                            const RowScales<SG>& sc) {
+    const float4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    if constexpr (SG == 1) {
+        float4_t t = zero;
+#pragma unroll
+        for (int st = 0; st < 4; ++st) t = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[st], unpack8_vec(wq[st]), t, 0, 0, 0);
+        acc += sc.get(0) * t;
+    } else {
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+            const float4_t t = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[st], unpack8_vec(wq[st]), zero, 0, 0, 0);
+            acc += sc.get(st) * t;
+        }
+    }
 }
 
-__device__ __forceinline__ void scale_add(float4_t& acc, const float4_t& t, u32x2_t scale_bits) {
-    acc[0] += half_bits_to_float(static_cast<uint16_t>(scale_bits[0] & 0xFFFFu)) * t[0];
-    acc[1] += half_bits_to_float(static_cast<uint16_t>(scale_bits[0] >> 16)) * t[1];
-    acc[2] += half_bits_to_float(static_cast<uint16_t>(scale_bits[1] & 0xFFFFu)) * t[2];
-    acc[3] += half_bits_to_float(static_cast<uint16_t>(scale_bits[1] >> 16)) * t[3];
+// Stores of a lane's four results (tokens 4*chunk..+3 of one output row): the fp16 hidden value
+// of the gate/up pair, or the weighted fp32 contribution (and, for a single slot, the reduce).
+__device__ __forceinline__ void store_hidden(const SegGateUpArgs& gu, const float4_t& gate, const float4_t& up,
+                                             int first, int token0, int count, int row) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        if (token0 + v < count) {
+            gu.hidden[static_cast<size_t>(first + token0 + v) * gu.I + row] =
+                float_to_half_bits(clamped_swiglu(gate[v], up[v], gu.limit));
+        }
+    }
 }
 
-// One workgroup = (R consecutive 16-row tiles, one segment). Lane l supplies weight row l%16 of
-// each tile / token l%16 and the 8-column chunk l/16 of each 32-column MFMA step; it ends up
-// holding output rows 4*(l/16)..+3 of token l%16 for each tile. The activation fragments of a
+__device__ __forceinline__ void store_contrib(const SegDownArgs& dn, const float4_t& acc, int first, int token0,
+                                              int count, int row, bool unit_weight) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        if (token0 + v >= count) continue;
+        const int position = first + token0 + v;
+        const float w = unit_weight ? 1.0f : dn.weight[position];
+        const float value = w * acc[v];
+        const size_t out_row = dn.out_row != nullptr ? dn.out_row[position] : position;
+        dn.contrib[out_row * dn.H + row] = value;
+        if (dn.fused_out != nullptr) {
+            // the reduce over a single slot, with its two roundings kept apart (no fused
+            // multiply-add): the stored fp32 contribution, then one fp16 rounding of the sum
+            const size_t at = static_cast<size_t>(position) * dn.H + row;
+            const float start = dn.fused_initial != nullptr ? half_bits_to_float(dn.fused_initial[at]) : 0.0f;
+            float product = value;
+            asm volatile("" : "+v"(product));   // keeps the multiply out of an fma with the add
+            dn.fused_out[at] = float_to_half_bits(start + product);
+        }
+    }
+}
+
+// One workgroup = (R consecutive 16-row tiles, one segment). The activation fragments of a
 // 128-column group are loaded once and used by all R tiles (and both matrices of gate/up).
-template <bool GATE_UP, int R, int WK, int D>
+template <bool GATE_UP, int R, int WK, int D, int SG>
 __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegDownArgs dn) {
     constexpr int NM = GATE_UP ? 2 : 1;
     const SegmentList& seg = GATE_UP ? gu.seg : dn.seg;
@@ -231,8 +329,8 @@ __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegD
         sm[NM - 1] = as_global<uint16_t>(e.w3_scale);
     }
 
-    // A padded token column repeats the segment's last live position: always a valid row, and
-    // its products land in output columns the store below never writes.
+    // A padded token row repeats the segment's last live position: always a valid row, and
+    // its products land in results the stores below never write.
     const int position = first + (n < count ? n : count - 1);
     const AEON_GLOBAL uint16_t* xrow;
     if (GATE_UP) {
@@ -254,7 +352,7 @@ __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegD
     // buffer is refilled for the group D steps ahead as soon as its MFMAs have been issued, so
     // every wave keeps D*NM*R KiB of HBM reads outstanding while it computes.
     u32x4_t wq[D][NM][R];
-    u32x2_t sc[D][NM][R];
+    RowScales<SG> sc[D][NM][R];
     half8_t xf[D][4];
     auto load_group = [&](int d, int g) {
 #pragma unroll
@@ -263,7 +361,7 @@ __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegD
             for (int r = 0; r < R; ++r) {
                 const size_t t = static_cast<size_t>(tile0 + r) * groups + g;
                 wq[d][m][r] = pm[m][t * 64 + lane];
-                sc[d][m][r] = *reinterpret_cast<const AEON_GLOBAL u32x2_t*>(sm[m] + t * 16 + chunk * 4);
+                sc[d][m][r].load(sm[m] + t * (16 * SG), n);
             }
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
@@ -280,7 +378,7 @@ __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegD
         for (int m = 0; m < NM; ++m)
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                scale_add(acc[m][r], mfma_group(wq[d][m][r], xf[d]), sc[d][m][r]);
+                mfma_scaled<SG>(acc[m][r], wq[d][m][r], xf[d], sc[d][m][r]);
             }
     };
 #pragma unroll
@@ -326,43 +424,14 @@ __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegD
                 for (int r = 0; r < R; ++r) acc[m][r] += partial[w][m][r][lane];
     }
 
-    if (n >= count) return;
+    // the lane holds tokens 4*chunk..+3 of output row (tile, n)
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const int row0 = (tile0 + r) * 16 + chunk * 4;
+        const int row = (tile0 + r) * 16 + n;
         if (GATE_UP) {
-            const float4_t& ga = acc[0][r];
-            const float4_t& up = acc[NM - 1][r];
-            uint2 packed;
-            packed.x = float_to_half_bits(clamped_swiglu(ga[0], up[0], gu.limit)) |
-                       (static_cast<uint32_t>(float_to_half_bits(
-                            clamped_swiglu(ga[1], up[1], gu.limit))) << 16);
-            packed.y = float_to_half_bits(clamped_swiglu(ga[2], up[2], gu.limit)) |
-                       (static_cast<uint32_t>(float_to_half_bits(
-                            clamped_swiglu(ga[3], up[3], gu.limit))) << 16);
-            *reinterpret_cast<uint2*>(gu.hidden + static_cast<size_t>(first + n) * gu.I + row0) = packed;
+            store_hidden(gu, acc[0][r], acc[NM - 1][r], first, chunk * 4, count, row);
         } else {
-            const float w = slot_mode && s == seg.slot_shared ? 1.0f : dn.weight[first + n];
-            const float4_t v = {w * acc[0][r][0], w * acc[0][r][1], w * acc[0][r][2], w * acc[0][r][3]};
-            const size_t out_row = dn.out_row != nullptr ? dn.out_row[first + n] : first + n;
-            *reinterpret_cast<float4_t*>(dn.contrib + out_row * dn.H + row0) = v;
-            if (dn.fused_out != nullptr) {
-                // the reduce over a single slot, with its two roundings kept apart (no fused
-                // multiply-add): the stored fp32 contribution, then one fp16 rounding of the sum
-                const size_t at = static_cast<size_t>(first + n) * dn.H + row0;
-                uint16_t o[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float start = dn.fused_initial != nullptr ? half_bits_to_float(dn.fused_initial[at + i]) : 0.0f;
-                    float product = v[i];
-                    asm volatile("" : "+v"(product));   // keeps the multiply out of an fma with the add
-                    o[i] = float_to_half_bits(start + product);
-                }
-                uint2 packed;
-                packed.x = o[0] | (static_cast<uint32_t>(o[1]) << 16);
-                packed.y = o[2] | (static_cast<uint32_t>(o[3]) << 16);
-                *reinterpret_cast<uint2*>(dn.fused_out + at) = packed;
-            }
+            store_contrib(dn, acc[0][r], first, chunk * 4, count, row, slot_mode && s == seg.slot_shared);
         }
     }
 }
@@ -382,7 +451,17 @@ __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegD
 // long list) streams its weights once per 32 positions instead of once per 16.
 static_assert(kWideSegTokens == kWideMaxTiles * kSegTokens, "segment length of the wide form");
 
-template <bool GATE_UP, int R, int D, int MT>
+// LDS of one wide-form workgroup: the activation ring (static) plus the scales of its four
+// waves' tiles over the whole of K (dynamic).
+constexpr size_t kWideActivationLdsBytes = 2 * kWideMaxTiles * 4 * 64 * 16;
+size_t seg_wide_scale_lds_bytes(bool gate_up, int row_tiles, int k_dim, int scales_per_group) {
+    return static_cast<size_t>(4) * (gate_up ? 2 : 1) * row_tiles * (k_dim / 128) * 32 * scales_per_group;
+}
+bool seg_wide_fits(bool gate_up, int row_tiles, int k_dim, int scales_per_group) {
+    return kWideActivationLdsBytes + seg_wide_scale_lds_bytes(gate_up, row_tiles, k_dim, scales_per_group) <= 65536;
+}
+
+template <bool GATE_UP, int R, int D, int MT, int SG>
 __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const SegDownArgs& dn, int s,
                                               int row_block, half8_t* xs, u32x4_t* scale_lds) {
     constexpr int NM = GATE_UP ? 2 : 1;
@@ -428,14 +507,14 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
         }
     }
 
-    const int tile_u4 = groups * 2;         // 32 bytes of scales per group
+    const int tile_u4 = groups * 2 * SG;    // 32 (SG 1) or 128 (SG 4) bytes of scales per group
     u32x4_t* my_scales = scale_lds + static_cast<size_t>(wave) * NM * R * tile_u4;
 #pragma unroll
     for (int m = 0; m < NM; ++m)
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const AEON_GLOBAL u32x4_t* src = reinterpret_cast<const AEON_GLOBAL u32x4_t*>(
-                sm[m] + static_cast<size_t>(tile0 + r) * groups * 16);
+                sm[m] + static_cast<size_t>(tile0 + r) * groups * (16 * SG));
             for (int i = lane; i < tile_u4; i += 64) my_scales[(m * R + r) * tile_u4 + i] = src[i];
         }
 
@@ -485,25 +564,27 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
     // fragment of group g+1 (fetched D steps ago) into the other LDS buffer, then request group
     // g+D's weights and group g+1+D's fragment. One barrier per group: buffer (g+1)&1 was last
     // read in step g-1, before that step's barrier.
-    const u32x2_t* scale_rows = reinterpret_cast<const u32x2_t*>(my_scales) + chunk;
+    const uint16_t* scale_halves = reinterpret_cast<const uint16_t*>(my_scales);
     auto step = [&](int d, int g, bool refill) {
         half8_t xf[MT][4];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int st = 0; st < 4; ++st) xf[mt][st] = *slot(g & 1, mt, st);
-        // The K steps run outermost and the wave's tiles innermost, so that consecutive matrix
-        // instructions belong to different accumulators: a chain of dependent ones would hold
-        // the SIMD for the latency of each.
-        float4_t t[NM][R][MT];
+        // this lane's weight row of each tile: its scale(s) of the group, 2 or 8 bytes from LDS
+        RowScales<SG> sc[NM][R];
 #pragma unroll
         for (int m = 0; m < NM; ++m)
 #pragma unroll
             for (int r = 0; r < R; ++r)
+                sc[m][r].load_lds(scale_halves + ((m * R + r) * tile_u4 + g * 2 * SG) * 8, n);
+        // The K steps run outermost and the wave's tiles innermost, so that consecutive matrix
+        // instructions belong to different accumulators: a chain of dependent ones would hold
+        // the SIMD for the latency of each.
+        const float4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
+        float4_t t[NM][R][MT];
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) t[m][r][mt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-        for (int st = 0; st < 4; ++st)
+        for (int st = 0; st < 4; ++st) {
 #pragma unroll
             for (int m = 0; m < NM; ++m)
 #pragma unroll
@@ -511,17 +592,20 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
                     const half8_t a = unpack8_vec(wq[d][m][r][st]);
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt)
-                        t[m][r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, xf[mt][st], t[m][r][mt], 0, 0, 0);
+                        t[m][r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                            xf[mt][st], a, (SG == 4 || st == 0) ? zero : t[m][r][mt], 0, 0, 0);
                 }
+            if (SG == 4 || st == 3) {
+                // one scale per row: the four steps have chained into t; four per row: every
+                // step's product takes the step's scale. fp32 either way.
 #pragma unroll
-        for (int m = 0; m < NM; ++m)
+                for (int m = 0; m < NM; ++m)
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                // scales of (tile, group): 16 rows x 2 bytes; this lane's rows are 4*chunk..+3
-                const u32x2_t sc = scale_rows[((m * R + r) * tile_u4 + g * 2) * 2];
+                    for (int r = 0; r < R; ++r)
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) scale_add(acc[m][r][mt], t[m][r][mt], sc);
+                        for (int mt = 0; mt < MT; ++mt) acc[m][r][mt] += sc[m][r].get(SG == 4 ? st : 0) * t[m][r][mt];
             }
+        }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) *slot((g + 1) & 1, mt, wave) = xr[(d + 1) % D][mt];
         if (refill) {
@@ -545,30 +629,17 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
         if (g0 + D + d < groups) step(d, g0 + D + d, false);
     }
 
+    // the lane holds tokens 16*mt + 4*chunk..+3 of output row (tile, n)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-        const int token = mt * kSegTokens + n;
-        if (token >= count) continue;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int row0 = (tile0 + r) * 16 + chunk * 4;
+            const int row = (tile0 + r) * 16 + n;
             if (GATE_UP) {
-                const float4_t& ga = acc[0][r][mt];
-                const float4_t& up = acc[NM - 1][r][mt];
-                uint2 packed;
-                packed.x = float_to_half_bits(clamped_swiglu(ga[0], up[0], gu.limit)) |
-                           (static_cast<uint32_t>(float_to_half_bits(
-                                clamped_swiglu(ga[1], up[1], gu.limit))) << 16);
-                packed.y = float_to_half_bits(clamped_swiglu(ga[2], up[2], gu.limit)) |
-                           (static_cast<uint32_t>(float_to_half_bits(
-                                clamped_swiglu(ga[3], up[3], gu.limit))) << 16);
-                *reinterpret_cast<uint2*>(gu.hidden + static_cast<size_t>(first + token) * gu.I + row0) = packed;
+                store_hidden(gu, acc[0][r][mt], acc[NM - 1][r][mt], first, mt * kSegTokens + chunk * 4, count, row);
             } else {
-                const float w = slot_mode && s == seg.slot_shared ? 1.0f : dn.weight[first + token];
-                const float4_t& a4 = acc[0][r][mt];
-                const float4_t v = {w * a4[0], w * a4[1], w * a4[2], w * a4[3]};
-                const size_t out_row = dn.out_row != nullptr ? dn.out_row[first + token] : first + token;
-                *reinterpret_cast<float4_t*>(dn.contrib + out_row * dn.H + row0) = v;
+                store_contrib(dn, acc[0][r][mt], first, mt * kSegTokens + chunk * 4, count, row,
+                              slot_mode && s == seg.slot_shared);
             }
         }
     }
@@ -577,7 +648,7 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
 // Four waves per SIMD (128 registers a wave) is what hides the weight stream's latency for the
 // common one-tile segment; the rarer two-tile path is kept inside that budget by a shallower
 // prefetch ring rather than allowed to halve everyone's occupancy.
-template <bool GATE_UP, int R, int D>
+template <bool GATE_UP, int R, int D, int SG>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void a64_seg_wide_kernel(
     SegGateUpArgs gu, SegDownArgs dn) {
     __shared__ half8_t xs[2 * kWideMaxTiles * 4 * 64];
@@ -590,32 +661,41 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             const int id = seg.expert[s];
             if (id < 0 || id >= seg.slot_experts) return;
         }
-        seg_wide_item<GATE_UP, R, D, 1>(gu, dn, s, blockIdx.x, xs, scale_lds);
+        seg_wide_item<GATE_UP, R, D, 1, SG>(gu, dn, s, blockIdx.x, xs, scale_lds);
         return;
     }
     if (s >= *seg.total) return;
     if (seg.count[s] > kSegTokens) {
-        seg_wide_item<GATE_UP, R, (D > 2 ? 2 : D), 2>(gu, dn, s, blockIdx.x, xs, scale_lds);
+        seg_wide_item<GATE_UP, R, (SG == 4 ? 1 : D > 2 ? 2 : D), 2, SG>(gu, dn, s, blockIdx.x, xs, scale_lds);
     } else {
-        seg_wide_item<GATE_UP, R, D, 1>(gu, dn, s, blockIdx.x, xs, scale_lds);
+        seg_wide_item<GATE_UP, R, D, 1, SG>(gu, dn, s, blockIdx.x, xs, scale_lds);
+    }
+}
+
+template <bool GATE_UP, int R, int D, int SG>
+static void launch_seg_rds(const SegGateUpArgs& gu, const SegDownArgs& dn, int tiles, int capacity,
+                           int k_split, hipStream_t stream) {
+    const dim3 grid(tiles / R, capacity);
+    if (k_split == 0) {
+        const size_t scale_bytes = seg_wide_scale_lds_bytes(GATE_UP, R, GATE_UP ? gu.H : dn.I, SG);
+        a64_seg_wide_kernel<GATE_UP, R, D, SG>
+            <<<dim3(tiles / (4 * R), capacity), 256, scale_bytes, stream>>>(gu, dn);
+    } else if (k_split >= 4 && (GATE_UP ? gu.H : dn.I) >= 4 * 128) {
+        a64_seg_kernel<GATE_UP, R, 4, D, SG><<<grid, 256, 0, stream>>>(gu, dn);
+    } else if (k_split >= 2 && (GATE_UP ? gu.H : dn.I) >= 2 * 128) {
+        a64_seg_kernel<GATE_UP, R, 2, D, SG><<<grid, 128, 0, stream>>>(gu, dn);
+    } else {
+        a64_seg_kernel<GATE_UP, R, 1, D, SG><<<grid, 64, 0, stream>>>(gu, dn);
     }
 }
 
 template <bool GATE_UP, int R, int D>
 static void launch_seg_rd(const SegGateUpArgs& gu, const SegDownArgs& dn, int tiles, int capacity,
                           int k_split, hipStream_t stream) {
-    const dim3 grid(tiles / R, capacity);
-    if (k_split == 0) {
-        const int k_dim = GATE_UP ? gu.H : dn.I;
-        const size_t scale_bytes = static_cast<size_t>(4) * (GATE_UP ? 2 : 1) * R * (k_dim / 128) * 32;
-        a64_seg_wide_kernel<GATE_UP, R, D>
-            <<<dim3(tiles / (4 * R), capacity), 256, scale_bytes, stream>>>(gu, dn);
-    } else if (k_split >= 4 && (GATE_UP ? gu.H : dn.I) >= 4 * 128) {
-        a64_seg_kernel<GATE_UP, R, 4, D><<<grid, 256, 0, stream>>>(gu, dn);
-    } else if (k_split >= 2 && (GATE_UP ? gu.H : dn.I) >= 2 * 128) {
-        a64_seg_kernel<GATE_UP, R, 2, D><<<grid, 128, 0, stream>>>(gu, dn);
+    if ((GATE_UP ? gu.scales_per_group : dn.scales_per_group) == 4) {
+        launch_seg_rds<GATE_UP, R, D, 4>(gu, dn, tiles, capacity, k_split, stream);
     } else {
-        a64_seg_kernel<GATE_UP, R, 1, D><<<grid, 64, 0, stream>>>(gu, dn);
+        launch_seg_rds<GATE_UP, R, D, 1>(gu, dn, tiles, capacity, k_split, stream);
     }
 }
 
@@ -641,6 +721,10 @@ static void launch_seg(const SegGateUpArgs& gu, const SegDownArgs& dn, int tiles
     if (k_split == 0 && (direct || tiles % (4 * (row_tiles >= 2 ? 2 : 1)) != 0)) {
         k_split = 1;  // the wide form needs a segment list and whole workgroups of tiles
     }
+    if (k_split == 0 && row_tiles >= 2 && tiles % 2 == 0 &&
+        !seg_wide_fits(GATE_UP, 2, GATE_UP ? gu.H : dn.I, GATE_UP ? gu.scales_per_group : dn.scales_per_group)) {
+        row_tiles = 1;  // two row tiles per wave would not fit their scales into LDS
+    }
     // Two row tiles per wave is the most the 128-register budget of the wide form carries.
     if (row_tiles >= 2 && tiles % 2 == 0) {
         launch_seg_r<GATE_UP, 2>(gu, dn, tiles, capacity, k_split, depth, stream);
@@ -653,6 +737,10 @@ int launch_seg_gate_up(const SegGateUpArgs& a, int k_split, int row_tiles, int d
     AEON_REQUIRE(a.H % 128 == 0 && a.I % 16 == 0 && a.x_stride % 8 == 0, AEON_ERR_INVALID_ARGUMENT,
                  "gate/up segments: need H%%128==0, I%%16==0 and an activation pitch that keeps "
                  "rows 16-byte aligned (H=%d I=%d pitch=%ld)", a.H, a.I, a.x_stride);
+    AEON_REQUIRE(a.scales_per_group == 1 || a.scales_per_group == 4, AEON_ERR_INVALID_ARGUMENT,
+                 "gate/up segments: %d scales per 128 columns (1 or 4)", a.scales_per_group);
+    AEON_REQUIRE(k_split != 0 || seg_wide_fits(true, 1, a.H, a.scales_per_group), AEON_ERR_INVALID_ARGUMENT,
+                 "gate/up segments: the scales of %d columns do not fit the wide form's LDS", a.H);
     if (a.seg.capacity <= 0) return AEON_OK;
     launch_seg<true>(a, SegDownArgs{}, a.I / 16, a.seg.capacity, k_split, row_tiles, depth, stream);
     AEON_LAUNCH_CHECK();
@@ -662,6 +750,10 @@ int launch_seg_gate_up(const SegGateUpArgs& a, int k_split, int row_tiles, int d
 int launch_seg_down(const SegDownArgs& a, int k_split, int row_tiles, int depth, hipStream_t stream) {
     AEON_REQUIRE(a.I % 128 == 0 && a.H % 16 == 0, AEON_ERR_INVALID_ARGUMENT,
                  "down segments: need I%%128==0 and H%%16==0 (H=%d I=%d)", a.H, a.I);
+    AEON_REQUIRE(a.scales_per_group == 1 || a.scales_per_group == 4, AEON_ERR_INVALID_ARGUMENT,
+                 "down segments: %d scales per 128 columns (1 or 4)", a.scales_per_group);
+    AEON_REQUIRE(k_split != 0 || seg_wide_fits(false, 1, a.I, a.scales_per_group), AEON_ERR_INVALID_ARGUMENT,
+                 "down segments: the scales of %d columns do not fit the wide form's LDS", a.I);
     if (a.seg.capacity <= 0) return AEON_OK;
     launch_seg<false>(SegGateUpArgs{}, a, a.H / 16, a.seg.capacity, k_split, row_tiles, depth, stream);
     AEON_LAUNCH_CHECK();
@@ -758,16 +850,17 @@ extern "C" int aeon_moe_accumulate_fixed_order_tokens(const float* d_contrib, in
 }
 
 extern "C" int aeon_a64_gemv(const void* d_x, int x_stride, const void* d_packed,
-                             const void* d_scale, void* d_out, int out_stride, int tokens, int N,
-                             int K, void* stream) {
+                             const void* d_scale, int scale_group, void* d_out, int out_stride,
+                             int tokens, int N, int K, void* stream) {
     const char* who = "aeon_a64_gemv";
     AEON_REQUIRE(d_x && d_packed && d_scale && d_out, AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
-    if (int rc = check_a64_shape(N, K, who)) return rc;
+    if (int rc = check_a64_shape(N, K, scale_group, who)) return rc;
     AEON_REQUIRE(tokens >= 1 && tokens <= 8, AEON_ERR_INVALID_ARGUMENT,
                  "%s: tokens=%d outside 1..8", who, tokens);
     AEON_REQUIRE(x_stride >= K && x_stride % 8 == 0 && out_stride >= N, AEON_ERR_INVALID_ARGUMENT,
                  "%s: bad row pitch (x_stride=%d out_stride=%d)", who, x_stride, out_stride);
     GemvArgs a{};
+    a.scales_per_group = scale_group == 32 ? 4 : 1;
     a.x = static_cast<const uint16_t*>(d_x);
     a.x_stride = x_stride;
     a.pa = static_cast<const uint4*>(d_packed);
@@ -782,17 +875,19 @@ extern "C" int aeon_a64_gemv(const void* d_x, int x_stride, const void* d_packed
 
 extern "C" int aeon_a64_dual_gemv(const void* d_x, int x_stride, const void* d_packed_a,
                                   const void* d_scale_a, const void* d_packed_b,
-                                  const void* d_scale_b, void* d_out_a, void* d_out_b,
-                                  int out_stride, int tokens, int N, int K, void* stream) {
+                                  const void* d_scale_b, int scale_group, void* d_out_a,
+                                  void* d_out_b, int out_stride, int tokens, int N, int K,
+                                  void* stream) {
     const char* who = "aeon_a64_dual_gemv";
     AEON_REQUIRE(d_x && d_packed_a && d_scale_a && d_packed_b && d_scale_b && d_out_a && d_out_b,
                  AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
-    if (int rc = check_a64_shape(N, K, who)) return rc;
+    if (int rc = check_a64_shape(N, K, scale_group, who)) return rc;
     AEON_REQUIRE(tokens >= 1 && tokens <= 8, AEON_ERR_INVALID_ARGUMENT,
                  "%s: tokens=%d outside 1..8", who, tokens);
     AEON_REQUIRE(x_stride >= K && x_stride % 8 == 0 && out_stride >= N, AEON_ERR_INVALID_ARGUMENT,
                  "%s: bad row pitch (x_stride=%d out_stride=%d)", who, x_stride, out_stride);
     GemvArgs a{};
+    a.scales_per_group = scale_group == 32 ? 4 : 1;
     a.x = static_cast<const uint16_t*>(d_x);
     a.x_stride = x_stride;
     a.pa = static_cast<const uint4*>(d_packed_a);
@@ -809,7 +904,7 @@ extern "C" int aeon_a64_dual_gemv(const void* d_x, int x_stride, const void* d_p
 }
 
 extern "C" int aeon_a64_expert_decode(const void* d_x, int tokens, const aeon_a64_expert* expert,
-                                      const float* d_route_weights, void* d_hidden,
+                                      int scale_group, const float* d_route_weights, void* d_hidden,
                                       float* d_contrib, const void* d_shared, void* d_out, int H,
                                       int I, float swiglu_limit, int use_mfma, void* stream) {
     const char* who = "aeon_a64_expert_decode";
@@ -820,6 +915,9 @@ extern "C" int aeon_a64_expert_decode(const void* d_x, int tokens, const aeon_a6
                  AEON_ERR_INVALID_ARGUMENT, "%s: the expert has a null sub-tensor", who);
     AEON_REQUIRE(H > 0 && I > 0 && H % 128 == 0 && I % 128 == 0, AEON_ERR_INVALID_ARGUMENT,
                  "%s: need H%%128==0 and I%%128==0 (H=%d I=%d)", who, H, I);
+    AEON_REQUIRE(scale_group == 128 || scale_group == 32, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: scale_group must be 128 or 32, not %d", who, scale_group);
+    const int per_group = scale_group == 32 ? 4 : 1;
     AEON_REQUIRE(tokens >= 1 && tokens <= (use_mfma ? kSegTokens : 8), AEON_ERR_INVALID_ARGUMENT,
                  "%s: tokens=%d outside 1..%d for this kernel family", who, tokens,
                  use_mfma ? kSegTokens : 8);
@@ -835,6 +933,7 @@ extern "C" int aeon_a64_expert_decode(const void* d_x, int tokens, const aeon_a6
         gu.seg.capacity = 1;
         gu.direct_expert = *expert;
         gu.direct_count = tokens;
+        gu.scales_per_group = per_group;
         if (int rc = launch_seg_gate_up(gu, 4, 1, 2, s)) return rc;
         SegDownArgs dn{};
         dn.hidden = static_cast<const uint16_t*>(d_hidden);
@@ -845,6 +944,7 @@ extern "C" int aeon_a64_expert_decode(const void* d_x, int tokens, const aeon_a6
         dn.seg.capacity = 1;
         dn.direct_expert = *expert;
         dn.direct_count = tokens;
+        dn.scales_per_group = per_group;
         dn.fused_out = static_cast<uint16_t*>(d_out);
         dn.fused_initial = static_cast<const uint16_t*>(d_shared);
         return launch_seg_down(dn, 4, 1, 2, s);   // the reduce over its one slot rides along
@@ -863,6 +963,7 @@ extern "C" int aeon_a64_expert_decode(const void* d_x, int tokens, const aeon_a6
         g.groups = H / 128;
         g.epilogue = 1;
         g.limit = swiglu_limit;
+        g.scales_per_group = per_group;
         if (int rc = launch_gemv<2>(g, s)) return rc;
         GemvArgs d{};
         d.x = static_cast<const uint16_t*>(d_hidden);
@@ -876,6 +977,7 @@ extern "C" int aeon_a64_expert_decode(const void* d_x, int tokens, const aeon_a6
         d.groups = I / 128;
         d.epilogue = 2;
         d.tok_weight = d_route_weights;
+        d.scales_per_group = per_group;
         if (int rc = launch_gemv<1>(d, s)) return rc;
     }
     return launch_token_reduce(d_contrib, tokens, 1, -1, static_cast<const uint16_t*>(d_shared), H,

@@ -43,6 +43,7 @@ struct SegGateUpArgs {
     float limit;
     aeon_a64_expert direct_expert;
     int direct_count;
+    int scales_per_group;     // 1: one fp16 scale per (row, 128 columns); 4: one per 32 columns
 };
 
 struct SegDownArgs {
@@ -60,12 +61,16 @@ struct SegDownArgs {
     // `out`; both [tokens][H]), which is the slot-ordered reduce over one slot.
     uint16_t* fused_out;
     const uint16_t* fused_initial;
+    int scales_per_group;     // as in SegGateUpArgs
 };
 
 // k_split: 1, 2 or 4 waves of a workgroup split K between them; 0 = the wide form (four waves,
 // each with its own row tiles, activations shared through LDS). row_tiles: 1 or 2 consecutive
 // 16-row tiles per wave share one read of the activations. depth: K groups of weights in
 // flight per wave (1..4).
+// The wide form keeps the scales of a workgroup's tiles over all of K in LDS: whether that fits
+// (64 KiB a workgroup, the activation ring included) for a launch of this shape.
+bool seg_wide_fits(bool gate_up, int row_tiles, int k_dim, int scales_per_group);
 int launch_seg_gate_up(const SegGateUpArgs& a, int k_split, int row_tiles, int depth, hipStream_t stream);
 int launch_seg_down(const SegDownArgs& a, int k_split, int row_tiles, int depth, hipStream_t stream);
 

@@ -57,7 +57,7 @@ __device__ __forceinline__ half8_t scaled_fragment(uint32_t word, half2_t scale2
 // Loads complete in issue order and every group issues the same number, so "group g+1 has
 // landed" is a bound on the count of outstanding loads; a group ends in a bare s_barrier (the
 // fences of __syncthreads would wait for every LDS-DMA request and drain the ring).
-template <bool GATE_UP, int R, int LIVE, int DEPTH>
+template <bool GATE_UP, int R, int LIVE, int DEPTH, int SG>
 __device__ __forceinline__ void grouped_run(const SegGateUpArgs& gu, const SegDownArgs& dn,
                                                  const aeon_a64_expert& e, int first, int count,
                                                  half8_t* xs_flat) {
@@ -93,7 +93,7 @@ __device__ __forceinline__ void grouped_run(const SegGateUpArgs& gu, const SegDo
     for (int r = 0; r < R; ++r) {
         const uint32_t t = static_cast<uint32_t>(tile0 + r) * groups;
         woff[r] = (t * 64 + lane) * 16;
-        soff[r] = (t * 16 + n) * 2;
+        soff[r] = (t * 16 + n) * 2 * SG;   // the row's scale(s) of group 0: 2 or 8 bytes
     }
     const AEON_GLOBAL char* xbase = as_global<char>(GATE_UP ? static_cast<const void*>(gu.x)
                                                             : static_cast<const void*>(dn.hidden));
@@ -121,7 +121,10 @@ __device__ __forceinline__ void grouped_run(const SegGateUpArgs& gu, const SegDo
             for (int mt = 0; mt < LIVE; ++mt) acc[m][r][mt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
     u32x4_t wq[STAGES][NM][R];
-    uint16_t sc[STAGES][NM][R];
+    // the row's scale of the group, or its four (one per MFMA step): the step's weights are
+    // multiplied by the step's scale in fp16, one rounding per weight either way
+    using RowScales = std::conditional_t<SG == 4, u32x2_t, uint16_t>;
+    RowScales sc[STAGES][NM][R];
 #define AEON_FULL_ISSUE(g_, stage_)                                                                 \
     do {                                                                                            \
         const int gi_ = (g_) < groups ? (g_) : groups - 1;                                          \
@@ -136,15 +139,20 @@ __device__ __forceinline__ void grouped_run(const SegGateUpArgs& gu, const SegDo
             _Pragma("unroll") for (int r = 0; r < R; ++r) {                                         \
                 wq[stage_][m][r] = *(const AEON_GLOBAL u32x4_t*)(                                   \
                     pm[m] + (woff[r] + static_cast<uint32_t>(gi_) * 1024u));                        \
-                sc[stage_][m][r] = *(const AEON_GLOBAL uint16_t*)(                                  \
-                    sm[m] + (soff[r] + static_cast<uint32_t>(gi_) * 32u));                          \
+                sc[stage_][m][r] = *(const AEON_GLOBAL RowScales*)(                                 \
+                    sm[m] + (soff[r] + static_cast<uint32_t>(gi_) * (32u * SG)));                   \
             }                                                                                       \
         }                                                                                           \
     } while (0)
 
-    auto scale_pair = [](uint16_t bits) {
+    auto scale_pair = [](const RowScales& row, int st) {
         union { uint16_t u; half_t h; } v;
-        v.u = bits;
+        if constexpr (SG == 4) {
+            const uint32_t w = row[st >> 1];
+            v.u = static_cast<uint16_t>((st & 1) ? (w >> 16) : (w & 0xFFFFu));
+        } else {
+            v.u = row;
+        }
         return half2_t{v.h, v.h};
     };
     // B fragment of block i (token tile i % LIVE, MFMA step i / LIVE) of a ring slot.
@@ -167,7 +175,7 @@ __device__ __forceinline__ void grouped_run(const SegGateUpArgs& gu, const SegDo
 #pragma unroll
     for (int m = 0; m < NM; ++m)
 #pragma unroll
-        for (int r = 0; r < R; ++r) a[0][m][r] = scaled_fragment(wq[0][m][r][0], scale_pair(sc[0][m][r]));
+        for (int r = 0; r < R; ++r) a[0][m][r] = scaled_fragment(wq[0][m][r][0], scale_pair(sc[0][m][r], 0));
     b[0] = fragment(0, 0);
     b[1] = fragment(0, 1);
     __builtin_amdgcn_sched_barrier(0);
@@ -199,8 +207,9 @@ __device__ __forceinline__ void grouped_run(const SegGateUpArgs& gu, const SegDo
                 if (f * LIVE / kFrags == mt) {
                     const int m = f / R, r = f % R;
                     a[(st + 1) % 2][m][r] =
-                        st < 3 ? scaled_fragment(wq[s][m][r][st < 3 ? st + 1 : 0], scale_pair(sc[s][m][r]))
-                               : scaled_fragment(wq[sn][m][r][0], scale_pair(sc[sn][m][r]));
+                        st < 3 ? scaled_fragment(wq[s][m][r][st < 3 ? st + 1 : 0],
+                                                 scale_pair(sc[s][m][r], st < 3 ? st + 1 : 0))
+                               : scaled_fragment(wq[sn][m][r][0], scale_pair(sc[sn][m][r], 0));
                 }
             }
         };
@@ -277,7 +286,7 @@ __device__ __forceinline__ void grouped_run(const SegGateUpArgs& gu, const SegDo
     }
 }
 
-template <bool GATE_UP, int R>
+template <bool GATE_UP, int R, int SG>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void a64_grouped_kernel(
     SegGateUpArgs gu, SegDownArgs dn) {
     const SegmentList& seg = GATE_UP ? gu.seg : dn.seg;
@@ -294,17 +303,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     const int live_tiles = (count + 15) >> 4;
     if (live_tiles > 6) {
-        grouped_run<GATE_UP, R, 8, 1>(gu, dn, e, first, count, xs);
+        grouped_run<GATE_UP, R, 8, 1, SG>(gu, dn, e, first, count, xs);
     } else if (live_tiles > 4) {
-        grouped_run<GATE_UP, R, 6, 1>(gu, dn, e, first, count, xs);
+        grouped_run<GATE_UP, R, 6, 1, SG>(gu, dn, e, first, count, xs);
     } else if (live_tiles > 3) {
-        grouped_run<GATE_UP, R, 4, 3>(gu, dn, e, first, count, xs);
+        grouped_run<GATE_UP, R, 4, 3, SG>(gu, dn, e, first, count, xs);
     } else if (live_tiles > 2) {
-        grouped_run<GATE_UP, R, 3, 3>(gu, dn, e, first, count, xs);
+        grouped_run<GATE_UP, R, 3, 3, SG>(gu, dn, e, first, count, xs);
     } else if (live_tiles > 1) {
-        grouped_run<GATE_UP, R, 2, 3>(gu, dn, e, first, count, xs);
+        grouped_run<GATE_UP, R, 2, 3, SG>(gu, dn, e, first, count, xs);
     } else {
-        grouped_run<GATE_UP, R, 1, 3>(gu, dn, e, first, count, xs);
+        grouped_run<GATE_UP, R, 1, 3, SG>(gu, dn, e, first, count, xs);
     }
 }
 
@@ -315,7 +324,13 @@ int launch_grouped_gate_up(const SegGateUpArgs& a, hipStream_t stream) {
     AEON_REQUIRE(a.seg.total != nullptr, AEON_ERR_INVALID_ARGUMENT,
                  "grouped gate/up: needs a position-tile list");
     if (a.seg.capacity <= 0) return AEON_OK;
-    a64_grouped_kernel<true, 2><<<dim3(a.I / 128, a.seg.capacity), 256, 0, stream>>>(a, SegDownArgs{});
+    AEON_REQUIRE(a.scales_per_group == 1 || a.scales_per_group == 4, AEON_ERR_INVALID_ARGUMENT,
+                 "grouped gate/up: %d scales per 128 columns (1 or 4)", a.scales_per_group);
+    if (a.scales_per_group == 4) {
+        a64_grouped_kernel<true, 2, 4><<<dim3(a.I / 128, a.seg.capacity), 256, 0, stream>>>(a, SegDownArgs{});
+    } else {
+        a64_grouped_kernel<true, 2, 1><<<dim3(a.I / 128, a.seg.capacity), 256, 0, stream>>>(a, SegDownArgs{});
+    }
     AEON_LAUNCH_CHECK();
     return AEON_OK;
 }
@@ -326,7 +341,13 @@ int launch_grouped_down(const SegDownArgs& a, hipStream_t stream) {
     AEON_REQUIRE(a.seg.total != nullptr, AEON_ERR_INVALID_ARGUMENT,
                  "grouped down: needs a position-tile list");
     if (a.seg.capacity <= 0) return AEON_OK;
-    a64_grouped_kernel<false, 4><<<dim3(a.H / 256, a.seg.capacity), 256, 0, stream>>>(SegGateUpArgs{}, a);
+    AEON_REQUIRE(a.scales_per_group == 1 || a.scales_per_group == 4, AEON_ERR_INVALID_ARGUMENT,
+                 "grouped down: %d scales per 128 columns (1 or 4)", a.scales_per_group);
+    if (a.scales_per_group == 4) {
+        a64_grouped_kernel<false, 4, 4><<<dim3(a.H / 256, a.seg.capacity), 256, 0, stream>>>(SegGateUpArgs{}, a);
+    } else {
+        a64_grouped_kernel<false, 4, 1><<<dim3(a.H / 256, a.seg.capacity), 256, 0, stream>>>(SegGateUpArgs{}, a);
+    }
     AEON_LAUNCH_CHECK();
     return AEON_OK;
 }

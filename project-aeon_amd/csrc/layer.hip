@@ -81,6 +81,9 @@ static int check_layer(const aeon_moe_layer* L, const char* who) {
                  AEON_ERR_INVALID_ARGUMENT, "%s: bad expert geometry (experts=%d top_k=%d)", who,
                  L->experts, L->top_k);
     AEON_REQUIRE(L->d_experts != nullptr, AEON_ERR_INVALID_ARGUMENT, "%s: null expert table", who);
+    AEON_REQUIRE(L->scale_group == 0 || L->scale_group == 128 || L->scale_group == 32,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: scale_group must be 128 (or 0) or 32, not %d", who,
+                 L->scale_group);
     return AEON_OK;
 }
 
@@ -154,16 +157,24 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     // activations through LDS, no K split). Few: split K four ways so the chip still fills.
     // Measured at H 7168 / I 2048: the gate/up launch is faster K-split up to batch 2 (17 live
     // lists) and wide from batch 4 (33) on; the down launch is faster wide at every batch.
-    const int split_gate = live_bound * (layer->intermediate / 16) >= 3072 ? 0 : 4;
-    const int split_down = live_bound * (layer->hidden / 16) >= 4000 ? 0 : 4;
+    // The wide form also has to hold its tiles' scales over all of K in LDS; where four scales
+    // per 128 columns of a long K do not fit, the K-split form (scales straight from memory)
+    // serves every batch.
+    const int per_group = layer->scale_group == 32 ? 4 : 1;
+    const int split_gate = live_bound * (layer->intermediate / 16) >= 3072 &&
+                                   seg_wide_fits(true, 1, layer->hidden, per_group) ? 0 : 4;
+    const int split_down = live_bound * (layer->hidden / 16) >= 4000 &&
+                                   seg_wide_fits(false, 1, layer->intermediate, per_group) ? 0 : 4;
     // Wide form: 64 gate/up rows or 128 down rows per workgroup and four (three) K groups of
     // weights in flight per wave measured best at batch 64 on both a concentrated and a spread
     // routing; more rows per workgroup save activation reads but leave fewer workgroups to
     // balance over the CUs.
     const int rows_gate = 1;
     const int rows_down = split_down == 0 ? (live_bound >= 32 ? 2 : 1) : 1;
-    const int depth_gate = split_gate == 0 ? 4 : 2;
-    const int depth_down = split_down == 0 ? 3 : 2;
+    // With four scales per 128 columns the wide kernels need more registers per group in flight;
+    // the depths below are the deepest rings that stay inside their 128-register budget.
+    const int depth_gate = split_gate == 0 ? (per_group == 4 ? 2 : 4) : 2;
+    const int depth_down = split_down == 0 ? (per_group == 4 && rows_down == 2 ? 2 : 3) : 2;
     // When both launches take the wide form, a segment holds two token tiles, so an expert with
     // 17..32 positions (and the always-on expert's list) streams its weights once, not twice.
     const bool both_wide = split_gate == 0 && split_down == 0 &&
@@ -206,6 +217,7 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     gu.H = layer->hidden;
     gu.I = layer->intermediate;
     gu.limit = layer->swiglu_limit;
+    gu.scales_per_group = per_group;
     if (stage_mask & AEON_STAGE_GATE_UP) {
         if (int rc = grouped ? launch_grouped_gate_up(gu, s)
                              : launch_seg_gate_up(gu, split_gate, rows_gate, depth_gate, s)) {
@@ -222,6 +234,7 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     dn.contrib = w.contrib;
     dn.H = layer->hidden;
     dn.I = layer->intermediate;
+    dn.scales_per_group = per_group;
     if (stage_mask & AEON_STAGE_DOWN) {
         if (int rc = grouped ? launch_grouped_down(dn, s)
                              : launch_seg_down(dn, split_down, rows_down, depth_down, s)) {

@@ -7,7 +7,10 @@
 // 128g + 32s + 8*chunk + 0..7, which is exactly the A operand of one
 // v_mfma_f32_16x16x32_f16 step (lane l supplies row l%16, k = 8*(l/16)..+7), so four
 // MFMA steps consume one tile with no cross-lane movement; a VALU GEMV reads the same
-// words against four 16-byte activation chunks. One fp16 scale per (row, 128-group).
+// words against four 16-byte activation chunks. Scales come in two forms, chosen when the
+// matrix is repacked: one fp16 per (row, 128-column group) at [tile][row%16] -- for payloads
+// whose four group-32 scales inside every 128 columns are bit-equal -- or all four kept, at
+// [tile][row%16][step], step s being the scale of columns 128g+32s..+31, i.e. of MFMA step s.
 #include "common.hpp"
 
 #include <cstring>
@@ -51,10 +54,19 @@ static bool a64_shape_ok(int N, int K, int rpw, int lpr) {
     return swizzle_shape_ok(N, K, rpw, lpr) && N % 16 == 0 && K % 128 == 0;
 }
 
+static bool scale_group_ok(int scale_group) { return scale_group == 128 || scale_group == 32; }
+
+// Index of the fp16 scale of (row, 128-column group, MFMA step) in the A64 scale array.
+__host__ __device__ static inline size_t a64_scale_index(int row, int group128, int step, int groups,
+                                                         int per_group) {
+    const size_t tile = static_cast<size_t>(row / 16) * groups + group128;
+    return per_group == 4 ? (tile * 16 + row % 16) * 4 + step : tile * 16 + row % 16;
+}
+
 __global__ __launch_bounds__(256) void a64_repack_kernel(
     const uint32_t* __restrict__ swz_packed, const uint16_t* __restrict__ swz_scale,
     uint4* __restrict__ a64_packed, uint16_t* __restrict__ a64_scale, int N, int K, int rpw,
-    int lpr, int* __restrict__ mismatch) {
+    int lpr, int per_group, int* __restrict__ mismatch) {
     // One thread per destination uint4: coalesced 16-byte stores; the four source words sit
     // in four different swizzled slots (one per 32-column step).
     const int groups = K / 128;
@@ -77,10 +89,17 @@ __global__ __launch_bounds__(256) void a64_repack_kernel(
     }
     a64_packed[idx] = make_uint4(words[0], words[1], words[2], words[3]);
     if (chunk == 0) {
-        a64_scale[tile * 16 + row % 16] = scales[0];
-        if (mismatch != nullptr &&
-            (scales[1] != scales[0] || scales[2] != scales[0] || scales[3] != scales[0])) {
-            atomicAdd(mismatch, 1);
+        if (per_group == 4) {
+            // 8 bytes per row: the row's four step scales side by side
+            const uint2 four = make_uint2(scales[0] | (static_cast<uint32_t>(scales[1]) << 16),
+                                          scales[2] | (static_cast<uint32_t>(scales[3]) << 16));
+            reinterpret_cast<uint2*>(a64_scale)[tile * 16 + row % 16] = four;
+        } else {
+            a64_scale[tile * 16 + row % 16] = scales[0];
+            if (mismatch != nullptr &&
+                (scales[1] != scales[0] || scales[2] != scales[0] || scales[3] != scales[0])) {
+                atomicAdd(mismatch, 1);
+            }
         }
     }
 }
@@ -135,18 +154,22 @@ extern "C" size_t aeon_a64_packed_bytes(int N, int K) {
     return static_cast<size_t>(N) * K / 2;
 }
 
-extern "C" size_t aeon_a64_scale_bytes(int N, int K) {
-    return static_cast<size_t>(N) * (K / 128) * 2;
+extern "C" size_t aeon_a64_scale_bytes(int N, int K, int scale_group) {
+    if (!scale_group_ok(scale_group)) return 0;
+    return static_cast<size_t>(N) * (K / 128) * 2 * (scale_group == 32 ? 4 : 1);
 }
 
 extern "C" int aeon_a64_repack_host(const uint32_t* swz_packed, const uint16_t* swz_scale, int N,
-                                    int K, int rpw, int lpr, uint32_t* a64_packed,
-                                    uint16_t* a64_scale) {
+                                    int K, int rpw, int lpr, int scale_group,
+                                    uint32_t* a64_packed, uint16_t* a64_scale) {
     AEON_REQUIRE(swz_packed && swz_scale && a64_packed && a64_scale, AEON_ERR_INVALID_ARGUMENT,
                  "aeon_a64_repack_host: null buffer");
     AEON_REQUIRE(a64_shape_ok(N, K, rpw, lpr), AEON_ERR_INVALID_ARGUMENT,
                  "aeon_a64_repack_host: needs N%%16==0, K%%128==0 and a valid swizzle cfg "
                  "(N=%d K=%d rpw=%d lpr=%d)", N, K, rpw, lpr);
+    AEON_REQUIRE(scale_group_ok(scale_group), AEON_ERR_INVALID_ARGUMENT,
+                 "aeon_a64_repack_host: scale_group must be 128 or 32, not %d", scale_group);
+    const int per_group = scale_group == 32 ? 4 : 1;
     const int groups = K / 128;
     const int iterations = (K / 32) / lpr;
     for (int row = 0; row < N; ++row) {
@@ -159,33 +182,38 @@ extern "C" int aeon_a64_repack_host(const uint32_t* swz_packed, const uint16_t* 
                     a64_packed[a64_slot(row, g, chunk, groups) * 4 + s] = swz_packed[slot * 4 + chunk];
                 }
             }
+            if (per_group == 4) {
+                for (int s = 0; s < 4; ++s) a64_scale[a64_scale_index(row, g, s, groups, 4)] = scales[s];
+                continue;
+            }
             AEON_REQUIRE(scales[1] == scales[0] && scales[2] == scales[0] && scales[3] == scales[0],
                          AEON_ERR_INVALID_ARGUMENT,
                          "aeon_a64_repack_host: row %d, 128-group %d carries four different "
-                         "group-32 scales; the wave64 packing stores one", row, g);
-            a64_scale[(static_cast<size_t>(row / 16) * groups + g) * 16 + row % 16] = scales[0];
+                         "group-32 scales; repack with scale_group 32 to keep them", row, g);
+            a64_scale[a64_scale_index(row, g, 0, groups, 1)] = scales[0];
         }
     }
     return AEON_OK;
 }
 
 extern "C" int aeon_a64_unrepack_host(const uint32_t* a64_packed, const uint16_t* a64_scale, int N,
-                                      int K, int rpw, int lpr, uint32_t* swz_packed,
-                                      uint16_t* swz_scale) {
+                                      int K, int rpw, int lpr, int scale_group,
+                                      uint32_t* swz_packed, uint16_t* swz_scale) {
     AEON_REQUIRE(swz_packed && swz_scale && a64_packed && a64_scale, AEON_ERR_INVALID_ARGUMENT,
                  "aeon_a64_unrepack_host: null buffer");
     AEON_REQUIRE(a64_shape_ok(N, K, rpw, lpr), AEON_ERR_INVALID_ARGUMENT,
                  "aeon_a64_unrepack_host: needs N%%16==0, K%%128==0 and a valid swizzle cfg "
                  "(N=%d K=%d rpw=%d lpr=%d)", N, K, rpw, lpr);
+    AEON_REQUIRE(scale_group_ok(scale_group), AEON_ERR_INVALID_ARGUMENT,
+                 "aeon_a64_unrepack_host: scale_group must be 128 or 32, not %d", scale_group);
+    const int per_group = scale_group == 32 ? 4 : 1;
     const int groups = K / 128;
     const int iterations = (K / 32) / lpr;
     for (int row = 0; row < N; ++row) {
         for (int g = 0; g < groups; ++g) {
-            const uint16_t scale =
-                a64_scale[(static_cast<size_t>(row / 16) * groups + g) * 16 + row % 16];
             for (int s = 0; s < 4; ++s) {
                 const size_t slot = swizzled_slot(row, g * 4 + s, rpw, lpr, iterations);
-                swz_scale[slot] = scale;
+                swz_scale[slot] = a64_scale[a64_scale_index(row, g, s, groups, per_group)];
                 for (int chunk = 0; chunk < 4; ++chunk) {
                     swz_packed[slot * 4 + chunk] = a64_packed[a64_slot(row, g, chunk, groups) * 4 + s];
                 }
@@ -196,19 +224,22 @@ extern "C" int aeon_a64_unrepack_host(const uint32_t* a64_packed, const uint16_t
 }
 
 extern "C" int aeon_a64_repack_device(const void* d_swz_packed, const void* d_swz_scale, int N,
-                                      int K, int rpw, int lpr, void* d_a64_packed,
-                                      void* d_a64_scale, int* d_mismatch, void* stream) {
+                                      int K, int rpw, int lpr, int scale_group,
+                                      void* d_a64_packed, void* d_a64_scale, int* d_mismatch,
+                                      void* stream) {
     AEON_REQUIRE(d_swz_packed && d_swz_scale && d_a64_packed && d_a64_scale,
                  AEON_ERR_INVALID_ARGUMENT, "aeon_a64_repack_device: null buffer");
     AEON_REQUIRE(a64_shape_ok(N, K, rpw, lpr), AEON_ERR_INVALID_ARGUMENT,
                  "aeon_a64_repack_device: needs N%%16==0, K%%128==0 and a valid swizzle cfg "
                  "(N=%d K=%d rpw=%d lpr=%d)", N, K, rpw, lpr);
+    AEON_REQUIRE(scale_group_ok(scale_group), AEON_ERR_INVALID_ARGUMENT,
+                 "aeon_a64_repack_device: scale_group must be 128 or 32, not %d", scale_group);
     const size_t total = static_cast<size_t>(N) * (K / 128) * 4;
     const unsigned blocks = static_cast<unsigned>((total + 255) / 256);
     a64_repack_kernel<<<blocks, 256, 0, as_stream(stream)>>>(
         static_cast<const uint32_t*>(d_swz_packed), static_cast<const uint16_t*>(d_swz_scale),
         static_cast<uint4*>(d_a64_packed), static_cast<uint16_t*>(d_a64_scale), N, K, rpw, lpr,
-        d_mismatch);
+        scale_group == 32 ? 4 : 1, d_mismatch);
     AEON_LAUNCH_CHECK();
     return AEON_OK;
 }

@@ -4,8 +4,9 @@
 // key + (i+1)*golden; source word w of a matrix is the low or high half of draw w/2; the scale
 // of (row, 128-group) is draw row*(K/128)+g mapped to [0.005, 0.02] in fp64 and rounded to
 // fp16 (round to nearest even, done with integer arithmetic so host and device agree bit for
-// bit). The output is the `.aeon` swizzled payload with the group-128 scale replicated over
-// its four group-32 slots.
+// bit). The output is the `.aeon` swizzled payload, either with one scale per 128 columns
+// replicated over its four group-32 slots or (scale_group 32) with a scale of its own per
+// (row, 32-column group): draw row*(K/32)+group of the same stream.
 #include "common.hpp"
 
 namespace aeon355 {
@@ -52,6 +53,7 @@ __device__ static inline uint32_t permute_nibbles(uint32_t source) {
 
 __global__ __launch_bounds__(256) void synth_matrix_kernel(uint64_t packed_key, uint64_t scale_key,
                                                            int N, int K, int rpw, int lpr,
+                                                           int scale_group,
                                                            uint4* __restrict__ packed,
                                                            uint16_t* __restrict__ scale) {
     // one thread per swizzled slot = (row, 32-column group)
@@ -72,7 +74,9 @@ __global__ __launch_bounds__(256) void synth_matrix_kernel(uint64_t packed_key, 
                               permute_nibbles(static_cast<uint32_t>(d0 >> 32)),
                               permute_nibbles(static_cast<uint32_t>(d1)),
                               permute_nibbles(static_cast<uint32_t>(d1 >> 32)));
-    const uint64_t sd = stream_draw(scale_key, static_cast<uint64_t>(row) * (K / 128) + group / 4);
+    const uint64_t sd = scale_group == 32
+                            ? stream_draw(scale_key, static_cast<uint64_t>(row) * (K / 32) + group)
+                            : stream_draw(scale_key, static_cast<uint64_t>(row) * (K / 128) + group / 4);
     const double u = static_cast<double>(sd >> 11) * (1.0 / 9007199254740992.0);
     scale[slot] = positive_double_to_half_bits(0.005 + 0.015 * u);
 }
@@ -82,18 +86,20 @@ __global__ __launch_bounds__(256) void synth_matrix_kernel(uint64_t packed_key, 
 using namespace aeon355;
 
 extern "C" int aeon_synth_matrix_swizzled(uint64_t seed, int expert, int matrix, int N, int K,
-                                          int rpw, int lpr, void* d_packed, void* d_scale,
-                                          void* stream) {
+                                          int rpw, int lpr, int scale_group, void* d_packed,
+                                          void* d_scale, void* stream) {
     const char* who = "aeon_synth_matrix_swizzled";
     AEON_REQUIRE(d_packed && d_scale, AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
     AEON_REQUIRE(rpw > 0 && lpr > 0 && rpw * lpr == 32 && N > 0 && K > 0 && N % rpw == 0 &&
                      K % 128 == 0 && (K / 32) % lpr == 0 && matrix >= 0 && matrix <= 2,
                  AEON_ERR_INVALID_ARGUMENT, "%s: bad shape (N=%d K=%d rpw=%d lpr=%d matrix=%d)", who,
                  N, K, rpw, lpr, matrix);
+    AEON_REQUIRE(scale_group == 128 || scale_group == 32, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: scale_group must be 128 or 32, not %d", who, scale_group);
     const size_t slots = static_cast<size_t>(N) * (K / 32);
     synth_matrix_kernel<<<static_cast<unsigned>((slots + 255) / 256), 256, 0, as_stream(stream)>>>(
         stream_key(seed, matrix, expert), stream_key(seed, 8 + matrix, expert), N, K, rpw, lpr,
-        static_cast<uint4*>(d_packed), static_cast<uint16_t*>(d_scale));
+        scale_group, static_cast<uint4*>(d_packed), static_cast<uint16_t*>(d_scale));
     AEON_LAUNCH_CHECK();
     return AEON_OK;
 }

@@ -21,7 +21,8 @@ class MoeLayerStruct(C.Structure):
                 ("top_k", C.c_int), ("has_shared", C.c_int), ("swiglu_limit", C.c_float),
                 ("score_kind", C.c_int), ("routed_scaling_factor", C.c_float),
                 ("renormalize", C.c_int), ("d_router_weight", C.c_void_p),
-                ("d_router_bias", C.c_void_p), ("d_experts", C.c_void_p)]
+                ("d_router_bias", C.c_void_p), ("d_experts", C.c_void_p),
+                ("scale_group", C.c_int)]
 
 
 def stream_ptr():
@@ -30,16 +31,19 @@ def stream_ptr():
 
 class ExpertPool:
     """`slots` experts of shape (H, I) in the wave64 packing, 4096-byte aligned slots laid out
-    [W1 packed | W1 scale | W3 packed | W3 scale | W2 packed | W2 scale]."""
+    [W1 packed | W1 scale | W3 packed | W3 scale | W2 packed | W2 scale]. `scale_group` = columns
+    per fp16 scale: 128 (payloads whose group-32 scales repeat in fours) or 32 (all kept)."""
 
-    def __init__(self, slots, hidden, intermediate, device="cuda"):
+    def __init__(self, slots, hidden, intermediate, device="cuda", scale_group=128):
         self.slots, self.H, self.I = slots, hidden, intermediate
+        self.scale_group = scale_group
         lib = capi.lib()
         self.pb13 = lib.aeon_a64_packed_bytes(intermediate, hidden)
-        self.sb13 = lib.aeon_a64_scale_bytes(intermediate, hidden)
+        self.sb13 = lib.aeon_a64_scale_bytes(intermediate, hidden, scale_group)
         self.pb2 = lib.aeon_a64_packed_bytes(hidden, intermediate)
-        self.sb2 = lib.aeon_a64_scale_bytes(hidden, intermediate)
-        self.slot_bytes = lib.aeon_a64_slot_bytes(hidden, intermediate)
+        self.sb2 = lib.aeon_a64_scale_bytes(hidden, intermediate, scale_group)
+        self.slot_bytes = lib.aeon_a64_slot_bytes(hidden, intermediate, scale_group)
+        assert self.slot_bytes > 0
         self.payload_bytes = 2 * (self.pb13 + self.sb13) + self.pb2 + self.sb2
         self.buffer = torch.empty(slots * self.slot_bytes, dtype=torch.uint8, device=device)
         base = self.buffer.data_ptr()
@@ -47,7 +51,7 @@ class ExpertPool:
         view = capi.A64Expert()
         for s in range(slots):
             capi.call("aeon_a64_slot_views", C.c_void_p(base + s * self.slot_bytes), hidden,
-                      intermediate, C.byref(view))
+                      intermediate, scale_group, C.byref(view))
             table[s] = [view.w1_packed, view.w1_scale, view.w3_packed, view.w3_scale,
                         view.w2_packed, view.w2_scale]
         self.host_table = table
@@ -56,20 +60,19 @@ class ExpertPool:
 
     def load_catalog(self, catalog, layer, first=0, count=None, first_slot=0):
         """Experts [first, first+count) of `layer` of an opened `.aeon` expert catalog -> slots
-        first_slot.. of this pool (payload -> device staging -> wave64 repack). Returns
-        the number of 128-groups with unequal group-32 scales (must be 0)."""
+        first_slot.. of this pool (payload -> device staging -> wave64 repack). A pool with
+        scale_group 128 raises ValueError for a payload whose group-32 scales differ inside 128
+        columns."""
         count = self.slots - first_slot if count is None else count
         table = (capi.A64Expert * count)()
-        mismatches = C.c_long(0)
         capi.call("aeon_resident_load_layer", catalog, layer, first, count, self.H, self.I,
+                  self.scale_group,
                   C.c_void_p(self.buffer.data_ptr() + first_slot * self.slot_bytes),
-                  C.c_size_t((self.slots - first_slot) * self.slot_bytes), table,
-                  C.byref(mismatches))
+                  C.c_size_t((self.slots - first_slot) * self.slot_bytes), table)
         for i in range(count):
             got = [table[i].w1_packed, table[i].w1_scale, table[i].w3_packed, table[i].w3_scale,
                    table[i].w2_packed, table[i].w2_scale]
             assert got == [int(v) for v in self.host_table[first_slot + i]]
-        return mismatches.value
 
     def expert_struct(self, slot):
         return capi.A64Expert(*[int(v) for v in self.host_table[slot]])
@@ -81,7 +84,7 @@ class ExpertPool:
         shapes = ((I, H, CFG13), (I, H, CFG13), (H, I, CFG2))
         for j, ((p, s), (n, k, cfg)) in enumerate(zip(mats, shapes)):
             capi.call("aeon_a64_repack_device", capi.vp(p), capi.vp(s), n, k, cfg[0], cfg[1],
-                      C.c_void_p(int(self.host_table[slot, 2 * j])),
+                      self.scale_group, C.c_void_p(int(self.host_table[slot, 2 * j])),
                       C.c_void_p(int(self.host_table[slot, 2 * j + 1])), capi.vp(mismatch),
                       stream_ptr())
 
@@ -100,7 +103,7 @@ class ExpertPool:
         for s in range(self.slots):
             for m, ((p, sc), (n, k, cfg)) in enumerate(zip(tmp, shapes)):
                 capi.call("aeon_synth_matrix_swizzled", C.c_uint64(seed), first_expert_id + s, m, n,
-                          k, cfg[0], cfg[1], capi.vp(p), capi.vp(sc), stream_ptr())
+                          k, cfg[0], cfg[1], self.scale_group, capi.vp(p), capi.vp(sc), stream_ptr())
             self.load_swizzled(s, tmp, mismatch)
         return int(mismatch.item())
 
@@ -119,7 +122,7 @@ class MoeLayer:
                                   score_kind, routed_scaling_factor, int(renormalize),
                                   router_weight.data_ptr() if router_weight is not None else None,
                                   router_bias.data_ptr() if router_bias is not None else None,
-                                  pool.table.data_ptr())
+                                  pool.table.data_ptr(), pool.scale_group)
         self.workspace = None
         self.workspace_tokens = 0
 

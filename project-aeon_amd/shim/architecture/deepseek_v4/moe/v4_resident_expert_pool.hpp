@@ -19,10 +19,13 @@ class V4ResidentExpertPool {
 public:
     // File names and format version are the reference's current artifact specification
     // (make_current_swizzled_artifact_spec: model_experts_swizzled.{aeon,index}, version 2,
-    // 4096-byte sectors).
+    // 4096-byte sectors). `scale_group` = columns per scale in the pool: 32 keeps every scale of
+    // the container (one per 32 columns, swizzled_expert_format.hpp:18-23 -- the default, right
+    // for any checkpoint); 128 stores one per 128 columns and refuses, with
+    // std::invalid_argument, a container whose four scales inside 128 columns are not all equal.
     V4ResidentExpertPool(const std::string& model_dir, int hidden, int intermediate,
-                         uint32_t format_version = 2, uint32_t sector_size = 4096)
-        : hidden_(hidden), intermediate_(intermediate) {
+                         uint32_t format_version = 2, uint32_t sector_size = 4096, int scale_group = 32)
+        : hidden_(hidden), intermediate_(intermediate), scale_group_(scale_group) {
         aeon355::throw_on_error(aeon_expert_catalog_open(
             (model_dir + "/model_experts_swizzled.index").c_str(),
             (model_dir + "/model_experts_swizzled.aeon").c_str(), format_version, sector_size, &catalog_));
@@ -30,10 +33,11 @@ public:
         uint32_t version = 0;
         aeon355::throw_on_error(
             aeon_expert_catalog_info(catalog_, &layers_, &experts_per_layer_, &payload, &version));
-        slot_bytes_ = aeon_a64_slot_bytes(hidden, intermediate);
+        slot_bytes_ = aeon_a64_slot_bytes(hidden, intermediate, scale_group);
         if (slot_bytes_ == 0) {
             close();
-            throw std::invalid_argument("V4ResidentExpertPool: hidden/intermediate must be multiples of 128");
+            throw std::invalid_argument("V4ResidentExpertPool: hidden/intermediate must be multiples of 128 "
+                                        "and scale_group 32 or 128");
         }
         try {
             const size_t layer_bytes = slot_bytes_ * experts_per_layer_;
@@ -42,16 +46,9 @@ public:
                                 sizeof(aeon_a64_expert) * experts_per_layer_ * layers_));
             std::vector<aeon_a64_expert> host(experts_per_layer_);
             for (uint32_t l = 0; l < layers_; ++l) {
-                long mismatches = 0;
                 aeon355::throw_on_error(aeon_resident_load_layer(
-                    catalog_, l, 0, experts_per_layer_, hidden, intermediate,
-                    static_cast<char*>(pool_) + l * layer_bytes, layer_bytes, host.data(), &mismatches));
-                if (mismatches != 0) {
-                    throw std::invalid_argument(
-                        "V4ResidentExpertPool: layer " + std::to_string(l) + " has " +
-                        std::to_string(mismatches) + " 128-column groups whose group-32 scales differ; "
-                        "the wave64 packing stores one scale per group (use the `.aeon` entry points)");
-                }
+                    catalog_, l, 0, experts_per_layer_, hidden, intermediate, scale_group,
+                    static_cast<char*>(pool_) + l * layer_bytes, layer_bytes, host.data()));
                 CHECK_HIP(hipMemcpy(tables_ + static_cast<size_t>(l) * experts_per_layer_, host.data(),
                                     sizeof(aeon_a64_expert) * experts_per_layer_, hipMemcpyHostToDevice));
             }
@@ -68,6 +65,8 @@ public:
     uint32_t layers() const { return layers_; }
     uint32_t experts_per_layer() const { return experts_per_layer_; }
     size_t resident_bytes() const { return slot_bytes_ * experts_per_layer_ * layers_; }
+    // What aeon_moe_layer::scale_group has to say for a layer over this pool's tables.
+    int scale_group() const { return scale_group_; }
     // Device table of layer l: experts_per_layer() entries.
     const aeon_a64_expert* table(uint32_t layer) const {
         if (layer >= layers_) throw std::out_of_range("V4ResidentExpertPool: layer past the catalog");
@@ -84,7 +83,7 @@ private:
         catalog_ = nullptr;
     }
 
-    int hidden_, intermediate_;
+    int hidden_, intermediate_, scale_group_;
     aeon_expert_catalog* catalog_ = nullptr;
     uint32_t layers_ = 0, experts_per_layer_ = 0;
     size_t slot_bytes_ = 0;

@@ -9,7 +9,8 @@ experts can be produced in HBM and any one of them regenerated here for checking
 Weights are defined in the *source* layout of aeon_w4a16_swizzle.hpp:45-85: packed [N][K/8]
 u32 with column k in nibble k%8 (value q in 0..15, weight q-8), one fp16 scale per
 (row, 128-column group) uniform in [0.005, 0.02] -- replicated over the four group-32 slots
-of the `.aeon` payload.
+of the `.aeon` payload -- or, with scale_group 32, one per (row, 32-column group) as the
+reference's format stores them (swizzled_expert_format.hpp:18-23).
 """
 import numpy as np
 
@@ -62,18 +63,19 @@ def normal(key, count):
     return np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * np.pi * u2)
 
 
-def expert_matrix_source(seed, expert, matrix, N, K):
-    """(packed [N*K/8] u32, scale128 [N][K/128] fp16) of one matrix in the source layout.
+def expert_matrix_source(seed, expert, matrix, N, K, scale_group=128):
+    """(packed [N*K/8] u32, scale [N][K/scale_group] fp16) of one matrix in the source layout.
     Word w takes the low or high 32 bits of draw w//2; the scale of (row, g) is draw
-    row*(K/128)+g of the matrix's scale stream mapped to [0.005, 0.02] and rounded to fp16."""
+    row*(K/scale_group)+g of the matrix's scale stream mapped to [0.005, 0.02] and rounded to
+    fp16."""
     words = N * K // 8
     u = draws(stream_key(seed, matrix, expert), 0, (words + 1) // 2)
     packed = np.empty(2 * u.size, dtype=np.uint32)
     packed[0::2] = (u & np.uint64(0xFFFFFFFF)).astype(np.uint32)
     packed[1::2] = (u >> np.uint64(32)).astype(np.uint32)
     packed = packed[:words]
-    s = uniform01(draws(stream_key(seed, STREAM_SCALE + matrix, expert), 0, N * (K // 128)))
-    scale = (0.005 + 0.015 * s).astype(np.float16).reshape(N, K // 128)
+    s = uniform01(draws(stream_key(seed, STREAM_SCALE + matrix, expert), 0, N * (K // scale_group)))
+    scale = (0.005 + 0.015 * s).astype(np.float16).reshape(N, K // scale_group)
     return packed, scale
 
 

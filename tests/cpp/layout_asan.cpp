@@ -30,15 +30,23 @@ int main() {
         if (aeon_swizzle_w4a16(src.get(), ssrc.get(), swz.get(), sswz.get(), N, K, rpw, lpr)) return fail("swizzle", N, K);
         if (aeon_unswizzle_w4a16(swz.get(), sswz.get(), back.get(), sback.get(), N, K, rpw, lpr)) return fail("unswizzle", N, K);
         if (std::memcmp(src.get(), back.get(), words * 4) || std::memcmp(ssrc.get(), sback.get(), scales * 2)) return fail("round trip", N, K);
-        const size_t pb = aeon_a64_packed_bytes(N, K), sb = aeon_a64_scale_bytes(N, K);
-        std::unique_ptr<uint8_t[]> a64p(new uint8_t[pb]), a64s(new uint8_t[sb]);
-        if (aeon_a64_repack_host(swz.get(), sswz.get(), N, K, rpw, lpr, reinterpret_cast<uint32_t*>(a64p.get()),
-                                 reinterpret_cast<uint16_t*>(a64s.get()))) return fail("repack", N, K);
-        std::unique_ptr<uint32_t[]> swz2(new uint32_t[words]);
-        std::unique_ptr<uint16_t[]> sswz2(new uint16_t[scales]);
-        if (aeon_a64_unrepack_host(reinterpret_cast<const uint32_t*>(a64p.get()), reinterpret_cast<const uint16_t*>(a64s.get()),
-                                   N, K, rpw, lpr, swz2.get(), sswz2.get())) return fail("unrepack", N, K);
-        if (std::memcmp(swz.get(), swz2.get(), words * 4) || std::memcmp(sswz.get(), sswz2.get(), scales * 2)) return fail("repack round trip", N, K);
+        // both scale groupings of the wave64 packing on exact-size buffers (the replicated
+        // scales above are a valid input for either)
+        for (const int scale_group : {128, 32}) {
+            const size_t pb = aeon_a64_packed_bytes(N, K), sb = aeon_a64_scale_bytes(N, K, scale_group);
+            std::unique_ptr<uint8_t[]> a64p(new uint8_t[pb]), a64s(new uint8_t[sb]);
+            if (aeon_a64_repack_host(swz.get(), sswz.get(), N, K, rpw, lpr, scale_group,
+                                     reinterpret_cast<uint32_t*>(a64p.get()),
+                                     reinterpret_cast<uint16_t*>(a64s.get()))) return fail("repack", N, K);
+            std::unique_ptr<uint32_t[]> swz2(new uint32_t[words]);
+            std::unique_ptr<uint16_t[]> sswz2(new uint16_t[scales]);
+            if (aeon_a64_unrepack_host(reinterpret_cast<const uint32_t*>(a64p.get()),
+                                       reinterpret_cast<const uint16_t*>(a64s.get()), N, K, rpw, lpr,
+                                       scale_group, swz2.get(), sswz2.get())) return fail("unrepack", N, K);
+            if (std::memcmp(swz.get(), swz2.get(), words * 4) || std::memcmp(sswz.get(), sswz2.get(), scales * 2)) {
+                return fail("repack round trip", N, K);
+            }
+        }
     }
     std::printf("ok\n");
     return 0;

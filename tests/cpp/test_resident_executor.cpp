@@ -29,12 +29,12 @@ static DeviceExpert make_expert(int id) {
     const int shape[3][4] = {{kIntermediate, kHidden, 4, 8}, {kIntermediate, kHidden, 4, 8}, {kHidden, kIntermediate, 8, 4}};
     for (int m = 0; m < 3; ++m) {
         aeon355::throw_on_error(aeon_synth_matrix_swizzled(77, id, m, shape[m][0], shape[m][1], shape[m][2],
-                                                           shape[m][3], e.payload + off[m][0],
+                                                           shape[m][3], 128, e.payload + off[m][0],
                                                            e.payload + off[m][1], nullptr));
         GATE_HIP(hipMalloc(&e.a64[2 * m], aeon_a64_packed_bytes(shape[m][0], shape[m][1])));
-        GATE_HIP(hipMalloc(&e.a64[2 * m + 1], aeon_a64_scale_bytes(shape[m][0], shape[m][1])));
+        GATE_HIP(hipMalloc(&e.a64[2 * m + 1], aeon_a64_scale_bytes(shape[m][0], shape[m][1], 128)));
         aeon355::throw_on_error(aeon_a64_repack_device(e.payload + off[m][0], e.payload + off[m][1],
-                                                       shape[m][0], shape[m][1], shape[m][2], shape[m][3],
+                                                       shape[m][0], shape[m][1], shape[m][2], shape[m][3], 128,
                                                        e.a64[2 * m], e.a64[2 * m + 1], nullptr, nullptr));
     }
     return e;
@@ -103,7 +103,7 @@ int main() {
         }
         d_tables[l] = to_device(table);
         layers[l] = aeon_moe_layer{kHidden, kIntermediate, kExperts, kSlots, 0, kLimit, AEON_ROUTER_SCORE_SIGMOID,
-                                   1.0f, 1, nullptr, nullptr, d_tables[l]};
+                                   1.0f, 1, nullptr, nullptr, d_tables[l], 128};
     }
     GATE_HIP(hipDeviceSynchronize());
 

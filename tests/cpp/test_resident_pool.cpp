@@ -56,37 +56,45 @@ int main() {
     const size_t off[3][2] = {{kL.w1_packed, kL.w1_scale}, {kL.w3_packed, kL.w3_scale}, {kL.w2_packed, kL.w2_scale}};
     const int shape[3][4] = {{kIntermediate, kHidden, 4, 8}, {kIntermediate, kHidden, 4, 8}, {kHidden, kIntermediate, 8, 4}};
 
-    // synthetic payloads on the device -> host -> container; the same payloads repacked directly
+    // synthetic payloads on the device -> host -> container; the same payloads repacked directly.
+    // Once with one scale per 128 columns (replicated over the payload's group-32 slots, one kept
+    // in the pool) and once with a scale of its own per 32 columns, all kept: the real format.
     std::vector<std::vector<uint8_t>> payloads;
-    std::vector<std::vector<aeon_a64_expert>> direct(kLayers);
     uint8_t* d_payload = nullptr;
     GATE_HIP(hipMalloc(&d_payload, kL.bytes));
+    const std::filesystem::path dir =
+        std::filesystem::temp_directory_path() / ("aeon_pool_gate_" + std::to_string(::getpid()));
+    std::filesystem::create_directories(dir);
+    for (const int scale_group : {32, 128}) {
+    payloads.clear();
+    std::vector<std::vector<aeon_a64_expert>> direct(kLayers);
     for (int l = 0; l < kLayers; ++l)
         for (int e = 0; e < kExperts; ++e) {
             void* a64[6];
             for (int m = 0; m < 3; ++m) {
                 aeon355::throw_on_error(aeon_synth_matrix_swizzled(31, 10 * l + e, m, shape[m][0], shape[m][1],
-                                                                   shape[m][2], shape[m][3], d_payload + off[m][0],
-                                                                   d_payload + off[m][1], nullptr));
+                                                                   shape[m][2], shape[m][3], scale_group,
+                                                                   d_payload + off[m][0], d_payload + off[m][1],
+                                                                   nullptr));
                 GATE_HIP(hipMalloc(&a64[2 * m], aeon_a64_packed_bytes(shape[m][0], shape[m][1])));
-                GATE_HIP(hipMalloc(&a64[2 * m + 1], aeon_a64_scale_bytes(shape[m][0], shape[m][1])));
+                GATE_HIP(hipMalloc(&a64[2 * m + 1], aeon_a64_scale_bytes(shape[m][0], shape[m][1], scale_group)));
                 aeon355::throw_on_error(aeon_a64_repack_device(d_payload + off[m][0], d_payload + off[m][1],
                                                                shape[m][0], shape[m][1], shape[m][2], shape[m][3],
-                                                               a64[2 * m], a64[2 * m + 1], nullptr, nullptr));
+                                                               scale_group, a64[2 * m], a64[2 * m + 1], nullptr,
+                                                               nullptr));
             }
             GATE_HIP(hipDeviceSynchronize());
             payloads.push_back(to_host(d_payload, kL.bytes));
             direct[l].push_back(aeon_a64_expert{a64[0], a64[1], a64[2], a64[3], a64[4], a64[5]});
         }
 
-    const std::filesystem::path dir =
-        std::filesystem::temp_directory_path() / ("aeon_pool_gate_" + std::to_string(::getpid()));
-    std::filesystem::create_directories(dir);
     write_container(dir, payloads, 2);
+    std::printf("  -- one scale per %d columns\n", scale_group);
 
     {
-        core::V4ResidentExpertPool pool(dir.string(), kHidden, kIntermediate);
+        core::V4ResidentExpertPool pool(dir.string(), kHidden, kIntermediate, 2, 4096, scale_group);
         expect(pool.layers() == kLayers && pool.experts_per_layer() == kExperts, "catalog shape read from the index");
+        expect(pool.scale_group() == scale_group, "the pool reports its scale grouping");
         bool same = true;
         for (int l = 0; l < kLayers; ++l) {
             const std::vector<aeon_a64_expert> table = to_host(pool.table(l), kExperts);
@@ -98,7 +106,7 @@ int main() {
                 for (int j = 0; j < 6; ++j) {
                     const int m = j / 2;
                     const size_t n = j % 2 == 0 ? aeon_a64_packed_bytes(shape[m][0], shape[m][1])
-                                                : aeon_a64_scale_bytes(shape[m][0], shape[m][1]);
+                                                : aeon_a64_scale_bytes(shape[m][0], shape[m][1], scale_group);
                     same = same && to_host(static_cast<const uint8_t*>(got[j]), n) ==
                                        to_host(static_cast<const uint8_t*>(want[j]), n);
                 }
@@ -110,7 +118,7 @@ int main() {
         std::vector<aeon_moe_layer> from_pool(kLayers), from_direct(kLayers);
         for (int l = 0; l < kLayers; ++l) {
             from_pool[l] = aeon_moe_layer{kHidden, kIntermediate, kExperts, kSlots, 0, 7.0f, AEON_ROUTER_SCORE_SIGMOID,
-                                          1.0f, 1, nullptr, nullptr, pool.table(l)};
+                                          1.0f, 1, nullptr, nullptr, pool.table(l), pool.scale_group()};
             from_direct[l] = from_pool[l];
             from_direct[l].d_experts = to_device(direct[l]);
         }
@@ -149,6 +157,7 @@ int main() {
         expect(identical, "executor over the loaded pool gives the bits of the directly built tables");
         expect(moved, "the routed experts changed the accumulator");
     }
+    }   // scale_group
 
     bool version_rejected = false, shape_rejected = false, missing_rejected = false, scales_rejected = false;
     try {
@@ -160,15 +169,22 @@ int main() {
     try {
         core::V4ResidentExpertPool pool((dir / "nowhere").string(), kHidden, kIntermediate);
     } catch (const std::runtime_error&) { missing_rejected = true; }
+    // the container on disk now holds the replicated payloads (the loop's last pass)
     payloads[3][kL.w3_scale + 2] ^= 0x04;  // one of four replicated group-32 scales no longer equal
     write_container(dir, payloads, 2);
     try {
-        core::V4ResidentExpertPool pool(dir.string(), kHidden, kIntermediate);
+        core::V4ResidentExpertPool pool(dir.string(), kHidden, kIntermediate, 2, 4096, /*scale_group=*/128);
     } catch (const std::invalid_argument&) { scales_rejected = true; }
+    bool scales_kept = false;
+    try {
+        core::V4ResidentExpertPool pool(dir.string(), kHidden, kIntermediate);   // default: all scales kept
+        scales_kept = pool.scale_group() == 32;
+    } catch (const std::exception&) {}
     expect(version_rejected, "an index of another format version throws std::runtime_error");
     expect(shape_rejected, "a shape whose payload size differs from the catalog's throws std::invalid_argument");
     expect(missing_rejected, "a missing container throws std::runtime_error");
-    expect(scales_rejected, "group-32 scales that differ inside a 128-group are refused, not averaged");
+    expect(scales_rejected, "group-32 scales that differ inside 128 columns are refused by a one-scale pool");
+    expect(scales_kept, "the same container loads into a pool that keeps every scale (the default)");
     std::filesystem::remove_all(dir);
     std::printf(g_failures == 0 ? "[PASS] resident pool\n" : "[FAIL] resident pool\n");
     return g_failures == 0 ? 0 : 1;

@@ -20,36 +20,40 @@ def u16p(a):
 
 class Matrix:
     """One int4 matrix in the three layouts: source, `.aeon` swizzled (group-32 scales) and the
-    wave64 packing (group-128 scales, via the library's own host repack)."""
+    wave64 packing (via the library's own host repack). `scale` is fp16 [N][K/scale_group]:
+    with scale_group 128 each scale is replicated over its four group-32 slots of the `.aeon`
+    payload and the packing stores one; with 32 every slot has its own and the packing keeps
+    all four."""
 
-    def __init__(self, packed_src, scale128, N, K, cfg):
-        self.N, self.K, self.cfg = N, K, cfg
+    def __init__(self, packed_src, scale, N, K, cfg, scale_group=128):
+        self.N, self.K, self.cfg, self.scale_group = N, K, cfg, scale_group
         self.src_packed = packed_src
-        self.scale128 = scale128
-        scale32 = np.ascontiguousarray(synth.scale32_from_scale128(scale128))
+        assert scale.shape == (N, K // scale_group)
+        scale32 = np.ascontiguousarray(synth.scale32_from_scale128(scale) if scale_group == 128 else scale)
+        self.scale32 = scale32
         self.swz_packed, self.swz_scale = orc.swizzle(packed_src, scale32.view(np.uint16).ravel(),
                                                       N, K, *cfg)
         self.a64_packed = np.empty(N * K // 8, dtype=np.uint32)
-        self.a64_scale = np.empty(N * K // 128, dtype=np.uint16)
+        self.a64_scale = np.empty(N * K // scale_group, dtype=np.uint16)
         capi.call("aeon_a64_repack_host", u32p(self.swz_packed), u16p(self.swz_scale), N, K,
-                  cfg[0], cfg[1], u32p(self.a64_packed), u16p(self.a64_scale))
+                  cfg[0], cfg[1], scale_group, u32p(self.a64_packed), u16p(self.a64_scale))
 
     def decode(self):
         return orc.swizzled_decode(self.swz_packed, self.swz_scale, self.N, self.K, *self.cfg)
 
 
-def synth_matrix(seed, expert, matrix, N, K):
+def synth_matrix(seed, expert, matrix, N, K, scale_group=128):
     cfg = CFG2 if matrix == synth.STREAM_W2 else CFG13
-    p, s = synth.expert_matrix_source(seed, expert, matrix, N, K)
-    return Matrix(p, s, N, K, cfg)
+    p, s = synth.expert_matrix_source(seed, expert, matrix, N, K, scale_group)
+    return Matrix(p, s, N, K, cfg, scale_group)
 
 
 class Expert:
-    def __init__(self, seed, expert, H, I):
-        self.H, self.I = H, I
-        self.w1 = synth_matrix(seed, expert, synth.STREAM_W1, I, H)
-        self.w3 = synth_matrix(seed, expert, synth.STREAM_W3, I, H)
-        self.w2 = synth_matrix(seed, expert, synth.STREAM_W2, H, I)
+    def __init__(self, seed, expert, H, I, scale_group=128):
+        self.H, self.I, self.scale_group = H, I, scale_group
+        self.w1 = synth_matrix(seed, expert, synth.STREAM_W1, I, H, scale_group)
+        self.w3 = synth_matrix(seed, expert, synth.STREAM_W3, I, H, scale_group)
+        self.w2 = synth_matrix(seed, expert, synth.STREAM_W2, H, I, scale_group)
 
     def ffn(self, x, limit, round_hidden=True, want_hidden=False):
         """Oracle FFN of fp16 activations x [tokens][H] -> float64 [tokens][H]."""

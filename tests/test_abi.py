@@ -23,7 +23,7 @@ def test_every_declared_symbol_is_exported():
     assert len(names) >= 30
     missing = [n for n in names if not hasattr(lib, n)]
     assert not missing, missing
-    assert lib.aeon_abi_version() == 1
+    assert lib.aeon_abi_version() == 2
 
 
 def test_header_compiles_as_c():
@@ -56,9 +56,11 @@ def test_argument_errors_without_device_work():
     with pytest.raises(ValueError, match="both a source and a destination"):
         capi.call("aeon_expert_permutation", one, 4, 6, 256, one, one, one, one, None, None)
     with pytest.raises(ValueError, match="wave64 packing"):
-        capi.call("aeon_a64_gemv", one, 256, one, one, one, 40, 1, 40, 256, None)
+        capi.call("aeon_a64_gemv", one, 256, one, one, 128, one, 40, 1, 40, 256, None)
     with pytest.raises(ValueError, match="tokens"):
-        capi.call("aeon_a64_gemv", one, 256, one, one, one, 64, 9, 64, 256, None)
+        capi.call("aeon_a64_gemv", one, 256, one, one, 128, one, 64, 9, 64, 256, None)
+    with pytest.raises(ValueError, match="scale_group"):
+        capi.call("aeon_a64_gemv", one, 256, one, one, 16, one, 64, 1, 64, 256, None)
     w2 = capi.W2Table()
     with pytest.raises(ValueError, match="expert_count"):
         capi.call("aeon_moe_fused_w2_accum", one, C.byref(w2), one, None, one, one, 0, 4096, 2048,
@@ -69,7 +71,7 @@ def test_argument_errors_without_device_work():
     with pytest.raises(ValueError, match="the sink holds"):
         capi.call("aeon_calibrate_mfma_f16", 1, 10, 4, one, C.c_size_t(512), None, None)
     from project_aeon_amd import moe
-    cfg = moe.MoeLayerStruct(7168, 2048, 256, 8, 1, 7.0, 1, 1.0, 1, None, None, 16)
+    cfg = moe.MoeLayerStruct(7168, 2048, 256, 8, 1, 7.0, 1, 1.0, 1, None, None, 16, 128)
     assert capi.lib().aeon_moe_layer_workspace_bytes(C.byref(cfg), 64) > 0
     assert capi.lib().aeon_moe_layer_workspace_bytes(C.byref(cfg), 1 << 28) == 0
     with pytest.raises(ValueError, match="32-bit positions"):

@@ -61,6 +61,12 @@ def experts():
     return [h.Expert(5, 100 * l + e, H, I) for l in range(LAYERS) for e in range(EXPERTS)]
 
 
+@pytest.fixture(scope="module")
+def experts32():
+    """The same experts with a scale of their own per 32 columns: what a real checkpoint holds."""
+    return [h.Expert(5, 100 * l + e, H, I, 32) for l in range(LAYERS) for e in range(EXPERTS)]
+
+
 def test_payload_layout_is_the_reference_constants():
     """At (4096, 2048) the offsets are the reference's hard-coded ones
     (swizzled_expert_format.hpp:11-30)."""
@@ -137,21 +143,25 @@ def test_catalog_rejects_what_the_reference_rejects(tmp_path, experts, fault):
 
 
 @pytest.mark.gpu
-def test_resident_load_matches_direct_repack(tmp_path, experts, orc):
+@pytest.mark.parametrize("scale_group", [128, 32])
+def test_resident_load_matches_direct_repack(tmp_path, experts, experts32, orc, scale_group):
     """Container -> device staging -> wave64 repack gives, bit for bit, the slots the
     host repack of the same matrices gives; a layer decode through the loaded pool is the one
-    through a pool uploaded directly."""
+    through a pool uploaded directly. With one scale per 128 columns (replicated in the payload)
+    and with every group-32 scale distinct and kept."""
     import torch
     from project_aeon_amd import moe, synth
+    experts = experts32 if scale_group == 32 else experts
+    ExpertPool = lambda slots, hh, ii: moe.ExpertPool(slots, hh, ii, scale_group=scale_group)
     payloads = [payload_of(e) for e in experts]
     index_path, experts_path = write_container(str(tmp_path), payloads, LAYERS, EXPERTS,
                                                order=[5, 3, 1, 0, 2, 4], pad=2)
     cat = open_catalog(index_path, experts_path)
     try:
         for layer in range(LAYERS):
-            pool = moe.ExpertPool(EXPERTS, H, I)
+            pool = ExpertPool(EXPERTS, H, I)
             pool.buffer.fill_(0x5A)
-            assert pool.load_catalog(cat, layer) == 0
+            pool.load_catalog(cat, layer)
             torch.cuda.synchronize()
             raw = pool.buffer.cpu().numpy()
             base = pool.buffer.data_ptr()
@@ -164,8 +174,8 @@ def test_resident_load_matches_direct_repack(tmp_path, experts, orc):
                     got = raw[at:at + w.nbytes]
                     assert got.tobytes() == w.tobytes(), (layer, s, j)
         # a partial range into the middle of a pool
-        pool = moe.ExpertPool(EXPERTS, H, I)
-        assert pool.load_catalog(cat, 1, first=1, count=2, first_slot=1) == 0
+        pool = ExpertPool(EXPERTS, H, I)
+        pool.load_catalog(cat, 1, first=1, count=2, first_slot=1)
         torch.cuda.synchronize()
         e = experts[EXPERTS + 2]
         at = int(pool.host_table[2, 4]) - pool.buffer.data_ptr()
@@ -174,10 +184,10 @@ def test_resident_load_matches_direct_repack(tmp_path, experts, orc):
         with pytest.raises(IndexError):
             pool.load_catalog(cat, 1, first=2, count=2)
         with pytest.raises(ValueError):
-            moe.ExpertPool(EXPERTS, 512, I).load_catalog(cat, 0)   # shape does not match payloads
+            ExpertPool(EXPERTS, 512, I).load_catalog(cat, 0)   # shape does not match payloads
         # decode through the loaded pool
-        pool = moe.ExpertPool(EXPERTS, H, I)
-        assert pool.load_catalog(cat, 0) == 0
+        pool = ExpertPool(EXPERTS, H, I)
+        pool.load_catalog(cat, 0)
         layer0 = moe.MoeLayer(pool, EXPERTS - 1, 2, True, 7.0)
         x = h.dev_half(synth.activations(5, 6, H))
         ids = h.to_dev(np.array([[0, 1], [1, 0], [0, 1], [1, 0], [0, 1], [1, 0]], dtype=np.int32))
@@ -193,9 +203,10 @@ def test_resident_load_matches_direct_repack(tmp_path, experts, orc):
 
 
 @pytest.mark.gpu
-def test_resident_load_counts_unequal_scales(tmp_path, experts):
-    """A payload whose four group-32 scales of one 128-group differ cannot be stored in the wave64
-    packing: the loader reports it instead of loading something else."""
+def test_resident_load_refuses_unequal_scales_in_a_one_scale_pool(tmp_path, experts):
+    """A payload whose four group-32 scales of one 128-column group differ cannot be stored with
+    one scale per 128 columns: the load fails (it does not return a pool that computes with
+    other weights), and the same container loads into a pool that keeps every scale."""
     from project_aeon_amd import moe
     payloads = [bytearray(payload_of(e)) for e in experts]
     lay = capi.PayloadLayout()
@@ -206,8 +217,31 @@ def test_resident_load_counts_unequal_scales(tmp_path, experts):
     cat = open_catalog(index_path, experts_path)
     try:
         pool = moe.ExpertPool(EXPERTS, H, I)
-        assert pool.load_catalog(cat, 0) == 1
-        assert pool.load_catalog(cat, 1) == 0
+        with pytest.raises(ValueError, match="scale_group 32"):
+            pool.load_catalog(cat, 0)
+        pool.load_catalog(cat, 1)                     # layer 1 is untouched
+        keep = moe.ExpertPool(EXPERTS, H, I, scale_group=32)
+        keep.buffer.fill_(0)                          # padding between sub-tensors compares equal
+        keep.load_catalog(cat, 0)
+        import torch
+        torch.cuda.synchronize()
+        # the flipped bit is in the pool: slot 1's W2 scales differ from a pool of the clean payload
+        clean = moe.ExpertPool(EXPERTS, H, I, scale_group=32)
+        clean.buffer.fill_(0)
+        os.makedirs(str(tmp_path / "clean"))
+        index2, experts2 = write_container(str(tmp_path / "clean"), [payload_of(x) for x in experts],
+                                           LAYERS, EXPERTS)
+        cat2 = open_catalog(index2, experts2)
+        try:
+            clean.load_catalog(cat2, 0)
+        finally:
+            capi.lib().aeon_expert_catalog_close(cat2)
+        torch.cuda.synchronize()
+        a, b = keep.buffer.cpu().numpy(), clean.buffer.cpu().numpy()
+        differing = np.flatnonzero(a != b)
+        assert differing.size == 1
+        at = int(keep.host_table[1, 5]) - keep.buffer.data_ptr()
+        assert at <= differing[0] < at + H * I // 16
     finally:
         capi.lib().aeon_expert_catalog_close(cat)
 

@@ -67,21 +67,24 @@ def test_config0_single_gemv_both_layouts(orc):
               capi.vp(out_swz), N, K, 4, 8, h.stream_ptr())
     out_a64 = torch.zeros(N, dtype=torch.float16, device="cuda")
     d_ap, d_as = h.dev_u32(m.a64_packed), h.dev_u16(m.a64_scale)
-    capi.call("aeon_a64_gemv", capi.vp(d_x), K, capi.vp(d_ap), capi.vp(d_as), capi.vp(out_a64), N,
-              1, N, K, h.stream_ptr())
+    capi.call("aeon_a64_gemv", capi.vp(d_x), K, capi.vp(d_ap), capi.vp(d_as), 128, capi.vp(out_a64),
+              N, 1, N, K, h.stream_ptr())
     for got in (out_swz, out_a64):
         g = got.cpu().numpy().astype(np.float64)
         assert np.abs(want).max() > 1.0
         assert h.rel_err(g, want) <= TOL
 
 
+@pytest.mark.parametrize("scale_group", [128, 32])
 @pytest.mark.parametrize("tokens", [1, 2, 3, 8])
 @pytest.mark.parametrize("N,K,matrix", [(2048, 7168, 0), (7168, 2048, 2), (64, 256, 0)])
-def test_a64_gemv_and_dual(orc, tokens, N, K, matrix):
+def test_a64_gemv_and_dual(orc, tokens, N, K, matrix, scale_group):
+    """scale_group 32: every (row, 32-column group) has a scale of its own, as in a real
+    `.aeon` payload (swizzled_expert_format.hpp:18-23)."""
     torch, h, capi = _setup()
     from project_aeon_amd import synth
-    ma = h.synth_matrix(3, 1, matrix, N, K)
-    mb = h.synth_matrix(3, 2, matrix, N, K)
+    ma = h.synth_matrix(3, 1, matrix, N, K, scale_group)
+    mb = h.synth_matrix(3, 2, matrix, N, K, scale_group)
     x = synth.activations(7, tokens, K)
     want_a = orc.swizzled_matvec(ma.swz_packed, ma.swz_scale, N, K, *ma.cfg, x.astype(np.float64))
     want_b = orc.swizzled_matvec(mb.swz_packed, mb.swz_scale, N, K, *mb.cfg, x.astype(np.float64))
@@ -89,12 +92,12 @@ def test_a64_gemv_and_dual(orc, tokens, N, K, matrix):
     pa, sa, pb, sb = (h.dev_u32(ma.a64_packed), h.dev_u16(ma.a64_scale), h.dev_u32(mb.a64_packed),
                       h.dev_u16(mb.a64_scale))
     single = torch.zeros(tokens, N, dtype=torch.float16, device="cuda")
-    capi.call("aeon_a64_gemv", capi.vp(d_x), K, capi.vp(pa), capi.vp(sa), capi.vp(single), N,
-              tokens, N, K, h.stream_ptr())
+    capi.call("aeon_a64_gemv", capi.vp(d_x), K, capi.vp(pa), capi.vp(sa), scale_group,
+              capi.vp(single), N, tokens, N, K, h.stream_ptr())
     oa = torch.zeros(tokens, N, dtype=torch.float16, device="cuda")
     ob = torch.zeros(tokens, N, dtype=torch.float16, device="cuda")
     capi.call("aeon_a64_dual_gemv", capi.vp(d_x), K, capi.vp(pa), capi.vp(sa), capi.vp(pb),
-              capi.vp(sb), capi.vp(oa), capi.vp(ob), N, tokens, N, K, h.stream_ptr())
+              capi.vp(sb), scale_group, capi.vp(oa), capi.vp(ob), N, tokens, N, K, h.stream_ptr())
     assert h.rel_err(single.cpu().numpy(), want_a) <= TOL
     assert h.rel_err(oa.cpu().numpy(), want_a) <= TOL
     assert h.rel_err(ob.cpu().numpy(), want_b) <= TOL
@@ -138,8 +141,11 @@ def test_gemv_rejects_bad_shapes():
         capi.call("aeon_w4a16_swizzled_gemv", None, capi.vp(t), capi.vp(t), capi.vp(t), 64, 256,
                   4, 8, None)
     with pytest.raises(ValueError):
-        capi.call("aeon_a64_gemv", capi.vp(t), 256, capi.vp(t), capi.vp(t), capi.vp(t), 64, 9, 64,
-                  256, None)
+        capi.call("aeon_a64_gemv", capi.vp(t), 256, capi.vp(t), capi.vp(t), 128, capi.vp(t), 64, 9,
+                  64, 256, None)
+    with pytest.raises(ValueError, match="scale_group"):
+        capi.call("aeon_a64_gemv", capi.vp(t), 256, capi.vp(t), capi.vp(t), 64, capi.vp(t), 64, 1,
+                  64, 256, None)
 
 
 @pytest.mark.parametrize("experts", [1, 6, 8])
@@ -228,15 +234,17 @@ def test_swizzled_expert_trio_reference_shapes(orc, experts):
     assert h.rel_err(acc32.cpu().numpy(), twice) <= TOL
 
 
+@pytest.mark.parametrize("scale_group", [128, 32])
 @pytest.mark.parametrize("use_mfma", [0, 1])
 @pytest.mark.parametrize("tokens", [1, 4, 8])
-def test_config1_one_expert_decode(orc, tokens, use_mfma):
+def test_config1_one_expert_decode(orc, tokens, use_mfma, scale_group):
     """BASELINE config 1: one routed expert, batch 1/4/8, H=7168, I=2048, clamp 7, output scaled
-    by a router weight in (0,1]."""
+    by a router weight in (0,1]; with one scale per 128 columns (the config) and with a scale
+    of its own per 32 columns (the `.aeon` format's grouping)."""
     torch, h, capi = _setup()
     from project_aeon_amd import synth
     H, I, limit = 7168, 2048, 7.0
-    e = h.Expert(0, 0, H, I)
+    e = h.Expert(0, 0, H, I, scale_group)
     de = h.DevExpert(e)
     x = synth.activations(0, tokens, H)
     w = synth.route_weights(0, tokens)
@@ -244,7 +252,7 @@ def test_config1_one_expert_decode(orc, tokens, use_mfma):
     hidden = torch.zeros(tokens, I, dtype=torch.float16, device="cuda")
     contrib = torch.zeros(tokens, H, dtype=torch.float32, device="cuda")
     out = torch.zeros(tokens, H, dtype=torch.float16, device="cuda")
-    capi.call("aeon_a64_expert_decode", capi.vp(d_x), tokens, C.byref(de.c), capi.vp(d_w),
+    capi.call("aeon_a64_expert_decode", capi.vp(d_x), tokens, C.byref(de.c), scale_group, capi.vp(d_w),
               capi.vp(hidden), capi.vp(contrib), None, capi.vp(out), H, I, C.c_float(limit),
               use_mfma, h.stream_ptr())
     want, want_hidden = e.ffn(x, limit, round_hidden=True, want_hidden=True)
@@ -263,12 +271,12 @@ def test_config1_one_expert_decode(orc, tokens, use_mfma):
     # out = half(float(start) + contrib), fp32 add, one rounding, no fused multiply-add
     start = h.dev_half(synth.activations(5, tokens, H))
     out2 = torch.zeros_like(out)
-    capi.call("aeon_a64_expert_decode", capi.vp(d_x), tokens, C.byref(de.c), capi.vp(d_w),
+    capi.call("aeon_a64_expert_decode", capi.vp(d_x), tokens, C.byref(de.c), scale_group, capi.vp(d_w),
               capi.vp(hidden), capi.vp(contrib), capi.vp(start), capi.vp(out2), H, I,
               C.c_float(limit), use_mfma, h.stream_ptr())
     assert torch.equal(out2, (start.float() + contrib).half())
     inplace = start.clone()
-    capi.call("aeon_a64_expert_decode", capi.vp(d_x), tokens, C.byref(de.c), capi.vp(d_w),
+    capi.call("aeon_a64_expert_decode", capi.vp(d_x), tokens, C.byref(de.c), scale_group, capi.vp(d_w),
               capi.vp(hidden), capi.vp(contrib), capi.vp(inplace), capi.vp(inplace), H, I,
               C.c_float(limit), use_mfma, h.stream_ptr())
     assert torch.equal(inplace, out2)

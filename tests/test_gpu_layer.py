@@ -19,15 +19,16 @@ def _setup():
     return torch, helpers, capi, moe, synth
 
 
-def test_device_generator_and_repack_bit_exact(orc):
+@pytest.mark.parametrize("scale_group", [128, 32])
+def test_device_generator_and_repack_bit_exact(orc, scale_group):
     """The device generator equals the host one, and the device repack equals the host repack,
-    for all three matrices of an expert at full size."""
+    for all three matrices of an expert at full size, in both scale groupings."""
     torch, h, capi, moe, synth = _setup()
     H, I = 7168, 2048
-    pool = moe.ExpertPool(2, H, I)
+    pool = moe.ExpertPool(2, H, I, scale_group=scale_group)
     assert pool.fill_synthetic(seed=5, first_expert_id=40) == 0
     torch.cuda.synchronize()
-    host = h.Expert(5, 41, H, I)
+    host = h.Expert(5, 41, H, I, scale_group)
     raw = pool.buffer.cpu().numpy()
     base = pool.slot_bytes
     for j, (m, which) in enumerate(((host.w1, "w1"), (host.w3, "w3"), (host.w2, "w2"))):
@@ -37,8 +38,8 @@ def test_device_generator_and_repack_bit_exact(orc):
     # the swizzled payload itself, for one matrix
     p = torch.empty(I * H // 2, dtype=torch.uint8, device="cuda")
     s = torch.empty(I * H // 32, dtype=torch.int16, device="cuda")
-    capi.call("aeon_synth_matrix_swizzled", C.c_uint64(5), 41, 1, I, H, 4, 8, capi.vp(p),
-              capi.vp(s), h.stream_ptr())
+    capi.call("aeon_synth_matrix_swizzled", C.c_uint64(5), 41, 1, I, H, 4, 8, scale_group,
+              capi.vp(p), capi.vp(s), h.stream_ptr())
     assert np.array_equal(p.cpu().numpy().view(np.uint32), host.w3.swz_packed)
     assert np.array_equal(s.cpu().numpy().view(np.uint16), host.w3.swz_scale)
 
@@ -56,8 +57,19 @@ def test_device_repack_flags_unequal_scales(orc):
     flag = torch.zeros(1, dtype=torch.int32, device="cuda")
     d_swp, d_sws = h.dev_u32(swp), h.dev_u16(sws)
     capi.call("aeon_a64_repack_device", capi.vp(d_swp), capi.vp(d_sws), N, K, 4,
-              8, capi.vp(out_p), capi.vp(out_s), capi.vp(flag), h.stream_ptr())
+              8, 128, capi.vp(out_p), capi.vp(out_s), capi.vp(flag), h.stream_ptr())
     assert int(flag.item()) == 2
+    # kept as they are, the same scales repack without a flag and equal the host repack
+    out_s4 = torch.empty(N * K // 32, dtype=torch.int16, device="cuda")
+    flag.zero_()
+    capi.call("aeon_a64_repack_device", capi.vp(d_swp), capi.vp(d_sws), N, K, 4,
+              8, 32, capi.vp(out_p), capi.vp(out_s4), capi.vp(flag), h.stream_ptr())
+    assert int(flag.item()) == 0
+    hp = np.empty(N * K // 8, dtype=np.uint32)
+    hs = np.empty(N * K // 32, dtype=np.uint16)
+    capi.call("aeon_a64_repack_host", h.u32p(swp), h.u16p(sws), N, K, 4, 8, 32, h.u32p(hp), h.u16p(hs))
+    assert np.array_equal(out_p.cpu().numpy().view(np.uint32), hp)
+    assert np.array_equal(out_s4.cpu().numpy().view(np.uint16), hs)
 
 
 @pytest.mark.parametrize("score_kind,k,scaling", [(1, 8, 1.0), (0, 6, 1.5)])
@@ -507,8 +519,10 @@ def test_random_layer_steps_against_oracle(orc):
     """Forty seeded random layer steps (hidden, intermediate, expert count, top-k, token count
     from 1 to 200, with and without an always-on expert, two ids out of range each): every token
     count class of the step -- direct slots, decode segments, grouped windows -- lands here with
-    shapes the other tests do not use. Three tokens of each against the oracle, to 6e-3 of the
-    peak; without an always-on expert the routed sum is added to what the output held."""
+    shapes the other tests do not use. Odd cases keep a scale of their own per 32 columns (the
+    `.aeon` format's grouping, four scales per 128 columns in the packing), even ones one per
+    128. Three tokens of each against the oracle, to 6e-3 of the peak; without an always-on
+    expert the routed sum is added to what the output held."""
     torch, h, capi, moe, synth = _setup()
     rng = np.random.default_rng(2024)
     for case in range(40):
@@ -519,7 +533,8 @@ def test_random_layer_steps_against_oracle(orc):
         T = int(rng.choice([1, 2, 3, 5, 16, 17, 33, 64, 100, 128, 129, 200]))
         shared = bool(rng.integers(0, 2))
         seed = 500 + case
-        pool = moe.ExpertPool(E + (1 if shared else 0), H, I)
+        scale_group = 32 if case % 2 else 128
+        pool = moe.ExpertPool(E + (1 if shared else 0), H, I, scale_group=scale_group)
         assert pool.fill_synthetic(seed=seed, first_expert_id=0) == 0
         layer = moe.MoeLayer(pool, E, k, shared, 7.0)
         ids = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
@@ -531,12 +546,12 @@ def test_random_layer_steps_against_oracle(orc):
         start = synth.activations(seed + 1, T, H).astype(np.float16)
         out = layer.routed(h.dev_half(x), h.to_dev(ids), h.to_dev(w),
                            out=h.to_dev(start.copy())).cpu().numpy()
-        what = (case, H, I, E, k, T, shared)
+        what = (case, H, I, E, k, T, shared, scale_group)
         assert np.isfinite(out).all(), what
         check = sorted({0, T // 2, T - 1})
         need = sorted({int(e) for t in check for e in ids[t] if 0 <= e < E})
-        experts = {e: h.Expert(seed, e, H, I) for e in need}
-        always = h.Expert(seed, E, H, I) if shared else None
+        experts = {e: h.Expert(seed, e, H, I, scale_group) for e in need}
+        always = h.Expert(seed, E, H, I, scale_group) if shared else None
         for t in check:
             keep = [s for s in range(k) if 0 <= ids[t, s] < E]
             contrib = np.zeros((len(keep), H))

@@ -193,6 +193,20 @@ def test_a64_address_is_a_bijection_and_matches_the_layout_statement(orc):
     bad[0, 1] ^= 1
     with pytest.raises(ValueError):
         orc.a64_pack(src, bad, N, K)
+    # four scales kept per 128 columns: same nibble addresses, scale of (row, 32-column group)
+    # at [tile][row%16][step]; a payload with a scale of its own per 32 columns decodes to the
+    # same matrix the `.aeon` reading gives
+    for r in range(N):
+        for c in range(0, K, 8):
+            pw, nib, si = orc.a64_address(K, r, c, 32)
+            assert (pw, nib) == orc.a64_address(K, r, c)[:2]
+            tile = (r // 16) * (K // 128) + c // 128
+            assert si == (tile * 16 + r % 16) * 4 + (c % 128) // 32
+    d32 = rng.uniform(0.005, 0.02, (N, K // 32)).astype(np.float16).view(np.uint16)
+    p4, s4 = orc.a64_pack(src, d32, N, K, 32)
+    assert np.array_equal(p4, p) and s4.size == N * K // 32
+    sw_p4, sw_s4 = orc.swizzle(src, d32.ravel(), N, K, 4, 8)
+    assert np.array_equal(orc.a64_decode(p4, s4, N, K, 32), orc.swizzled_decode(sw_p4, sw_s4, N, K, 4, 8))
 
 
 def test_sinkhorn_closed_forms(orc):
