@@ -242,6 +242,47 @@ def run_dropin(capi, moe, torch, np):
                               "weights_gbps": round(NE * expert_bytes / ms / 1e6, 1),
                               "ms": round(ms, 3),
                               "tflops": round(2.0 * draws * 3 * H * I / ms / 1e9, 1)})
+
+    # The same payloads on the resident path: re-swizzled once into the wave64 packing with all
+    # four group-32 scales kept (scale_group 32), then aeon_moe_layer_routed -- one device expert
+    # table for the whole layer, ids and permutation never leave the device.
+    NE = len(experts)
+    pool = moe.ExpertPool(NE, H, I, scale_group=32)
+    for slot, m in enumerate(experts):
+        pool.load_swizzled(slot, (m["w1"], m["w3"], m["w2"]))
+    torch.cuda.synchronize()
+    del experts
+    res["resident"] = []
+    for T, live in ((1, 64), (8, 64), (64, 64), (256, 64), (1024, 64), (256, 256)):
+        layer = moe.MoeLayer(pool, NE, K, False, limit)
+        rng = np.random.default_rng(T)
+        rot = []
+        for r in range(8):
+            if T == 1:
+                ids_h = np.array([[(K * (r + 1) + j) % live for j in range(K)]], dtype=np.int32)
+            else:
+                ids_h = np.stack([rng.permutation(live)[:K] for _ in range(T)]).astype(np.int32)
+            rot.append(torch.from_numpy(ids_h).cuda())
+        w = torch.full((T, K), 1.0 / K, device="cuda")
+        xin = (torch.rand(T, H, device="cuda") - 0.5).half()
+        outb = torch.zeros(T, H, dtype=torch.float16, device="cuda")
+
+        def step(i):
+            layer.routed(xin, rot[i % 8], w, out=outb)
+
+        settle(step, torch)
+        reps = 200 if T <= 64 else 20
+        a.record()
+        for i in range(reps):
+            step(i)
+        b.record()
+        torch.cuda.synchronize()
+        ms = a.elapsed_time(b) / reps
+        touched = np.mean([len(np.unique(r.cpu().numpy())) for r in rot])
+        res["resident"].append({"tokens": T, "experts_live": live, "distinct_experts": round(float(touched), 1),
+                                "ms": round(ms, 4), "us_per_token": round(ms * 1e3 / T, 2),
+                                "weights_gbps": round(touched * expert_bytes / ms / 1e6, 1),
+                                "tflops": round(2.0 * T * K * 3 * H * I / ms / 1e9, 1)})
     return res
 
 

@@ -229,6 +229,74 @@ def test_config2_moe_layer_decode_reduced_experts(orc, B):
     assert np.array_equal(out2.cpu().numpy(), out)
 
 
+@pytest.mark.parametrize("H,I,E,k,T,shared", [
+    (4096, 2048, 64, 6, 64, False),     # the checkpoint's own shape: wide decode segments
+    (4096, 2048, 64, 6, 1, False),      # one token: slots read directly, K-split kernels
+    (4096, 2048, 32, 6, 48, True),      # hot experts: two token tiles per segment (wide form)
+    (4096, 2048, 64, 6, 300, False),    # a prefill chunk: grouped windows
+    (7168, 2048, 24, 8, 64, True),      # K too long for the wide form's LDS: K-split at a batch
+])
+def test_group32_scales_on_the_resident_path(orc, H, I, E, k, T, shared):
+    """Experts with a scale of their own per 32 columns (the `.aeon` format's grouping,
+    swizzled_expert_format.hpp:18-23; the reference model is hidden 4096, intermediate 2048,
+    top-6) through aeon_moe_layer_routed with the four-scale packing. Sampled tokens against the
+    oracle to 6e-3 of the peak, every token finite, run twice for the same bits; the decode
+    steps are also held to the `.aeon`-layout trio on the same payloads, which applies the same
+    exact fp32 scale per 32 columns."""
+    torch, h, capi, moe, synth = _setup()
+    limit = 10.0
+    pool = moe.ExpertPool(E + (1 if shared else 0), H, I, scale_group=32)
+    assert pool.fill_synthetic(seed=90, first_expert_id=0) == 0
+    layer = moe.MoeLayer(pool, E, k, shared, limit)
+    rng = np.random.default_rng(T + E)
+    hot = E if T != 48 else 3
+    ids = np.stack([np.concatenate([rng.permutation(hot)[:min(k, hot)],
+                                    hot + rng.permutation(E - hot)[:k - min(k, hot)]])
+                    for _ in range(T)]).astype(np.int32)
+    w = synth.route_weights(90, T * k).reshape(T, k).astype(np.float32)
+    x = synth.activations(90, T, H)
+    d_x, d_ids, d_w = h.dev_half(x), h.to_dev(ids), h.to_dev(w)
+    out = layer.routed(d_x, d_ids, d_w).cpu().numpy()
+    assert np.isfinite(out).all()
+    assert np.array_equal(layer.routed(d_x, d_ids, d_w).cpu().numpy(), out)
+    sample = sorted({0, T // 2, T - 1})
+    needed = sorted({int(e) for t in sample for e in ids[t]})
+    experts = {e: h.Expert(90, e, H, I, 32) for e in needed}
+    always = h.Expert(90, E, H, I, 32) if shared else None
+    want = _oracle_layer(orc, h, experts, x[sample], ids[sample], w[sample], always, limit)
+    assert np.abs(want).max() > 0.5
+    assert np.abs(out[sample] - want).max() <= 6e-3 * np.abs(want).max()
+    # one-scale reading of the same experts is a different layer: the check is not vacuous
+    wrong = {e: h.Expert(90, e, H, I, 128) for e in needed[:1]}
+    assert np.abs(wrong[needed[0]].w1.decode() - experts[needed[0]].w1.decode()).max() > 1e-3
+    if T <= 64 and not shared:
+        # the `.aeon`-layout trio of one token on the same payloads
+        t = sample[-1]
+        w13, w2 = capi.W13Table(), capi.W2Table()
+        keep = []
+        for j in range(k):
+            e = experts[int(ids[t, j])]
+            dev = [h.dev_u32(e.w1.swz_packed), h.dev_u16(e.w1.swz_scale), h.dev_u32(e.w3.swz_packed),
+                   h.dev_u16(e.w3.swz_scale), h.dev_u32(e.w2.swz_packed), h.dev_u16(e.w2.swz_scale)]
+            keep.append(dev)
+            w13.w1[j], w13.s1[j], w13.w3[j], w13.s3[j] = (dev[0].data_ptr(), dev[1].data_ptr(),
+                                                          dev[2].data_ptr(), dev[3].data_ptr())
+            w2.w2[j], w2.s2[j] = dev[4].data_ptr(), dev[5].data_ptr()
+        hidden = torch.zeros(k, I, dtype=torch.float16, device="cuda")
+        contrib = torch.zeros(k, H, dtype=torch.float32, device="cuda")
+        trio = torch.zeros(H, dtype=torch.float16, device="cuda")
+        xt = d_x[t].contiguous()
+        wt = d_w[t].contiguous()
+        capi.call("aeon_moe_gemv_w13_swiglu", capi.vp(xt), C.byref(w13), capi.vp(hidden), None, I, k,
+                  I, H, 4, 8, C.c_float(limit), h.stream_ptr())
+        capi.call("aeon_moe_fused_w2_contrib", capi.vp(hidden), C.byref(w2), capi.vp(wt),
+                  capi.vp(contrib), k, H, I, 8, 4, h.stream_ptr())
+        capi.call("aeon_moe_accumulate_fixed_order", capi.vp(contrib), k, None, capi.vp(trio), H,
+                  h.stream_ptr())
+        trio = trio.cpu().numpy().astype(np.float64)
+        assert np.abs(trio - out[t]).max() <= 2e-3 * np.abs(trio).max()
+
+
 def test_config2_full_size_sampled(orc):
     """BASELINE config 2 as written: batch 64, top-8 of 256 experts + the always-on one, fp32
     router with sigmoid scores and bias, H=7168, I=2048. The oracle covers a sample of tokens
