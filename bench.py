@@ -424,17 +424,21 @@ def run_other_configs(pool, layer, moe, capi, synth, torch, np, H, I, E, K_TOP, 
         out = torch.empty(tokens, H, dtype=torch.float16, device="cuda")
         structs = [pool.expert_struct(s) for s in range(pool.slots)]
 
-        def expert(i):
-            capi.call("aeon_a64_expert_decode", capi.vp(x), tokens, C.byref(structs[i % pool.slots]),
-                      pool.scale_group, capi.vp(w), capi.vp(hidden), capi.vp(contrib), None, capi.vp(out), H, I,
-                      C.c_float(LIMIT), 1, moe.stream_ptr())
-
-        ms = timed(expert, reps)
+        # both kernel families: the VALU dual-GEMV pair (v_dot2, no matrix instruction: what
+        # the routed step uses for one or two tokens of an expert) and the MFMA segment kernels
         b1 = 3 * bm + tokens * H * 2 * 2
-        res["config1_one_expert"].append(
-            {"batch": tokens, "us": round(ms * 1e3, 2), "us_per_token": round(ms * 1e3 / tokens, 2),
-             "algorithmic_bytes": b1, "achieved_gbps": round(b1 / (ms * 1e-3) / 1e9, 1),
-             "frac_of_peak": round(b1 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+        for family, use_mfma in (("valu_gemv", 0), ("mfma_segment", 1)):
+            def expert(i, use_mfma=use_mfma):
+                capi.call("aeon_a64_expert_decode", capi.vp(x), tokens, C.byref(structs[i % pool.slots]),
+                          pool.scale_group, capi.vp(w), capi.vp(hidden), capi.vp(contrib), None,
+                          capi.vp(out), H, I, C.c_float(LIMIT), use_mfma, moe.stream_ptr())
+
+            ms = timed(expert, reps)
+            res["config1_one_expert"].append(
+                {"batch": tokens, "kernels": family, "us": round(ms * 1e3, 2),
+                 "us_per_token": round(ms * 1e3 / tokens, 2), "algorithmic_bytes": b1,
+                 "achieved_gbps": round(b1 / (ms * 1e-3) / 1e9, 1),
+                 "frac_of_peak": round(b1 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
     # config 4: 4 stacked layers (independent seeded weights), batch B, hyper-connection mix of 4
     # residual streams between layers
     layers, mixes = [layer], []
@@ -503,9 +507,11 @@ def main():
     ap.add_argument("--cpu-tokens", type=int, default=64,
                     help="tokens of the batch the CPU oracle is timed on")
     ap.add_argument("--no-prefill", action="store_true", help="skip the config-3 prefill leg")
-    ap.add_argument("--all-configs", action="store_true",
-                    help="also time configs 0 (single GEMV), 1 (one expert, batch 1/4/8) and 4 "
-                         "(4 stacked layers with the hyper-connection mix) into `other_configs`")
+    ap.add_argument("--no-all-configs", dest="all_configs", action="store_false",
+                    help="skip configs 0 (single GEMV), 1 (one expert, batch 1/4/8, both kernel "
+                         "families) and 4 (4 stacked layers with the hyper-connection mix), which "
+                         "the default run reports in `other_configs`")
+    ap.add_argument("--all-configs", dest="all_configs", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--router-bias-scale", type=float, default=1.0,
                     help="scale of the per-expert router bias in the headline leg (1 = BASELINE's "
                          "N(0, 0.1); 0 = no bias, the spread routing)")
@@ -524,8 +530,10 @@ def main():
     ap.add_argument("--chunk-sweep", action="store_true",
                     help="also time the routed step at 64..1024 tokens (uniform and Zipf routing) "
                          "into `chunk_sweep`")
-    ap.add_argument("--sweep", action="store_true",
-                    help="also report batch 1/8/32/64 in the `sweep` field")
+    ap.add_argument("--no-sweep", dest="sweep", action="store_false",
+                    help="skip the batch 1/8/32/64 sweep of config 2 the default run reports in `sweep`")
+    ap.add_argument("--sweep", dest="sweep", action="store_true", help=argparse.SUPPRESS)
+    ap.set_defaults(all_configs=True, sweep=True)
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU's share of the path and uses no second GPU "

@@ -69,6 +69,33 @@ class Expert:
                                    *self.w2.cfg, np.asarray(hidden, dtype=np.float64))
 
 
+class GeneratedExpert:
+    """The oracle's view of synthetic expert (seed, expert): its `.aeon` payload produced by the
+    device generator and copied back (the generator is held to the host one bit for bit by the
+    GPU suite), for tests that need many full-size experts and cannot afford the host generator.
+    Same ffn()/down() as Expert."""
+
+    def __init__(self, seed, expert, H, I, scale_group=128):
+        import torch
+        self.H, self.I = H, I
+        self.mats = []
+        for m, (n, k, cfg) in enumerate(((I, H, CFG13), (I, H, CFG13), (H, I, CFG2))):
+            p = torch.empty(n * k // 2, dtype=torch.uint8, device="cuda")
+            sc = torch.empty(n * k // 32, dtype=torch.int16, device="cuda")
+            capi.call("aeon_synth_matrix_swizzled", C.c_uint64(seed), expert, m, n, k, cfg[0], cfg[1],
+                      scale_group, capi.vp(p), capi.vp(sc), stream_ptr())
+            self.mats.append((p.cpu().numpy().view(np.uint32), sc.cpu().numpy().view(np.uint16)))
+
+    def ffn(self, x, limit, round_hidden=True, want_hidden=False):
+        w1, w3, w2 = self.mats
+        return orc.expert_ffn(w1, w3, w2, self.H, self.I, np.asarray(x, dtype=np.float64), limit,
+                              round_hidden=round_hidden, want_hidden=want_hidden)
+
+    def down(self, hidden):
+        p, sc = self.mats[2]
+        return orc.swizzled_matvec(p, sc, self.H, self.I, *CFG2, np.asarray(hidden, dtype=np.float64))
+
+
 def to_dev(a):
     import torch
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()

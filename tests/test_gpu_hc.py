@@ -155,11 +155,14 @@ def test_dynamic_mix_projection_norm_and_post(orc, tokens, H):
     assert torch.equal(first, hc.mixes)
 
 
-@pytest.mark.parametrize("B,H,I,E", [(64, 1024, 512, 16), (4, 7168, 2048, 12)])
+@pytest.mark.parametrize("B,H,I,E", [(64, 1024, 512, 16), (4, 7168, 2048, 12), (64, 7168, 2048, 256)])
 def test_config4_stacked_layers(orc, B, H, I, E):
     """Four MoE layers with independent seeded weights and the HC mix between them. Each layer is
     checked against the oracle on the device's own input to that layer and the device's routed
-    ids (the way a composed gate isolates one stage from the rounding of the ones before it)."""
+    ids (the way a composed gate isolates one stage from the rounding of the ones before it).
+    The last case is BASELINE config 4 as written: 4 x (256 + 1) resident experts (23 GB), batch
+    64; there the oracle takes three tokens of every layer and its experts' payloads come back
+    from the device generator."""
     torch, h, capi, moe, synth = _setup()
     k, limit, L = 8, 7.0, 4
     layers, mixes, host = [], [], []
@@ -184,9 +187,10 @@ def test_config4_stacked_layers(orc, B, H, I, E):
         res_in, x, y = res_in.cpu().numpy(), x.cpu().numpy(), y.cpu().numpy()
         ids, w, res_out = ids.cpu().numpy(), w.cpu().numpy(), res_out.cpu().numpy()
         pre, post, comb = orc.hc_sinkhorn(mix, np.ones(3), np.zeros(24), 4)
-        check = range(B) if H <= 1024 else range(min(B, 2))
-        experts = {int(e): h.Expert(11, 1000 * l + int(e), H, I) for t in check for e in ids[t]}
-        shared = h.Expert(11, 1000 * l + E, H, I)
+        check = range(B) if H <= 1024 else (range(min(B, 2)) if E < 256 else (0, B // 2, B - 1))
+        make = h.GeneratedExpert if E >= 256 else h.Expert
+        experts = {int(e): make(11, 1000 * l + int(e), H, I) for t in check for e in ids[t]}
+        shared = make(11, 1000 * l + E, H, I)
         for t in check:
             r = res_in[:, t, :].astype(np.float64)
             want_x = orc.hc_pre_combine(r, pre, H)
