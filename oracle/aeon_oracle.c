@@ -397,6 +397,12 @@ static double router_score(double logit, int score_kind) {
     return score_kind == 0 ? sqrt(softplus(logit)) : sigmoid(logit);
 }
 
+/* The fp64 scores the selection below compares, one per logit: for tests that need to know how
+ * close two candidates are. */
+void orc_router_scores(const double* logits, size_t n, int score_kind, double* scores) {
+    for (size_t i = 0; i < n; ++i) scores[i] = router_score(logits[i], score_kind);
+}
+
 void orc_router_topk(const double* logits, const double* bias, size_t experts,
                      size_t top_k, double scaling, int score_kind,
                      int bias_before_activation, int32_t* ids, double* weights) {

@@ -252,6 +252,15 @@ def topk_indices(scores, k):
     return ids
 
 
+def router_scores(logits, score_kind):
+    """The fp64 scores router_topk compares (before any bias)."""
+    l = np.ascontiguousarray(logits, dtype=np.float64)
+    out = np.empty(l.size, dtype=np.float64)
+    lib().orc_router_scores(_ptr(l, C.c_double), C.c_size_t(l.size), int(score_kind),
+                            _ptr(out, C.c_double))
+    return out.reshape(l.shape)
+
+
 def router_topk(logits, bias, top_k, scaling, score_kind, bias_before=False):
     l = np.ascontiguousarray(logits, dtype=np.float64)
     b = np.ascontiguousarray(bias, dtype=np.float64) if bias is not None else None

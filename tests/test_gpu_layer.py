@@ -111,6 +111,57 @@ def test_router_ids_bit_exact_on_identical_logits(orc, score_kind, k, scaling):
     assert np.array_equal(ids, table[tok].astype(np.int32))
 
 
+@pytest.mark.parametrize("score_kind,exact_from", [(1, 8), (0, 16)])
+def test_router_near_ties_order_like_the_oracle(orc, score_kind, exact_from, capsys):
+    """How far "ids bit-exact" reaches. The device scores and selects in fp64 with its own exp /
+    log1p / sqrt; the oracle with the host's. Two candidates whose biased scores differ by a few
+    fp64 units in the last place (relative 1e-16) can therefore be ordered differently. The
+    probes are built on the host: two live experts with random fp32 logits, the second's bias the
+    fp32 nearest the score difference, the first's a tiny fp32 that closes the remaining gap to
+    j units in the last place (a bias of magnitude 1e-9 has an fp32 spacing far below one fp64
+    unit at 1), j from -64 to 64; six other experts far below. From `exact_from` units on the
+    device must pick what the oracle picks, for every probe; below that the agreement is
+    printed (measured: 1 probe of 150 differs for sigmoid out to 4 units, 5 of 150 for
+    sqrt(softplus) at 0..1 units, one run with other draws showed single ones out to 6)."""
+    torch, h, capi, moe, synth = _setup()
+    rng = np.random.default_rng(3 + score_kind)
+    E, js = 8, [-64, -32, -16, -8, -4, -3, -2, -1, 0, 1, 2, 3, 4, 8, 16, 32, 64]
+    logits_rows, bias_rows, meta = [], [], []
+    while len(meta) < 150 * len(js):
+        la, lb = rng.normal(0, 2, 2).astype(np.float32)
+        sa, sb = orc.router_scores(np.array([la, lb], dtype=np.float64), score_kind)
+        bb = np.float32(sa - sb)
+        if not 1e-3 < abs(float(bb)) < 0.5:
+            continue
+        ulp = np.spacing(max(sa, sb + float(bb)))
+        pa, pb = (int(v) for v in rng.permutation(E)[:2])
+        for j in js:
+            logits = np.full(E, -30.0, dtype=np.float32)
+            bias = np.zeros(E, dtype=np.float32)
+            logits[pa], logits[pb] = la, lb
+            bias[pa], bias[pb] = np.float32((sb + float(bb) - sa) + j * ulp), bb
+            logits_rows.append(logits)
+            bias_rows.append(bias)
+            meta.append(j)
+    agree = {j: [0, 0] for j in js}
+    ids = torch.zeros(1, 1, dtype=torch.int32, device="cuda")
+    w = torch.zeros(1, 1, dtype=torch.float32, device="cuda")
+    for logits, bias, j in zip(logits_rows, bias_rows, meta):
+        oi, _ = orc.router_topk(logits.astype(np.float64), bias.astype(np.float64), 1, 1.0, score_kind)
+        d_l, d_b = h.to_dev(logits.reshape(1, E)), h.to_dev(bias)
+        capi.call("aeon_moe_router", capi.vp(d_l), capi.vp(d_b), None, None, capi.vp(w), capi.vp(ids),
+                  1, E, 1, C.c_float(1.0), 1, score_kind, h.stream_ptr())
+        agree[j][0] += int(ids.item() == oi[0])
+        agree[j][1] += 1
+    with capsys.disabled():
+        print("\n  near-tie agreement (units in the last place: agreed/probes), score kind %d: %s"
+              % (score_kind, ", ".join("%+d: %d/%d" % (j, a, n) for j, (a, n) in sorted(agree.items()))))
+    for j, (a, n) in agree.items():
+        if abs(j) >= exact_from:
+            assert a == n, (score_kind, j, a, n)
+    assert sum(a for a, _ in agree.values()) >= 0.97 * sum(n for _, n in agree.values())
+
+
 @pytest.mark.parametrize("T,H,E", [(5, 1024, 10), (33, 896, 6), (3, 7168, 258), (17, 200, 64)])
 def test_router_logits_at_expert_counts_not_divisible_by_four(orc, T, H, E):
     """aeon_router_logits where a weight row is not a whole number of 16-byte vectors (E % 4 != 0)
