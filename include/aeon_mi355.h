@@ -228,6 +228,31 @@ int aeon_router_logits(const void* d_x, int x_stride, const float* d_router_weig
                        float* d_logits, int tokens, int hidden, int experts, void* d_workspace,
                        size_t workspace_bytes, void* stream);
 
+/* The same logits from the gate as the checkpoint stores it: gemv_fp16_vec8_kernel + the
+ * widening of dispatch_router (src/platform/ops/gemv.hpp:72-110, layer/v4_layer_body_moe.hpp:
+ * 135-142). d_gate_weight fp16 [experts][hidden]; logits_half[t][e] = half(sum_h x[t][h] *
+ * w[e][h]) (fp32 accumulate, one rounding) and logits[t][e] = float(logits_half[t][e]).
+ * hidden % 128 == 0, experts % 16 == 0. */
+int aeon_router_logits_f16(const void* d_x, int x_stride, const void* d_gate_weight,
+                           void* d_logits_half, float* d_logits, int tokens, int hidden,
+                           int experts, void* stream);
+
+/* gemv_fp16_vec8_kernel launch, src/platform/ops/gemv.hpp:72-110, for `tokens` rows at once:
+ * y[t][o] = half(sum_i x[t][i] * w[o][i]), w fp16 [out_dim][in_dim] row-major, fp32 accumulate.
+ * in_dim % 128 == 0, out_dim % 16 == 0, x_stride % 8 == 0, y_stride % 4 == 0. */
+int aeon_dense_gemv_f16(const void* d_x, int x_stride, const void* d_weight, void* d_y,
+                        int y_stride, int tokens, int in_dim, int out_dim, void* stream);
+/* run_layer_body_moe_shared_expert, layer/v4_layer_body_moe.hpp:216-256 (oracle: dense_ffn,
+ * reference/dsv4_oracle.hpp:1708-1753), for `tokens` tokens in two launches: gate = half(W1 x),
+ * up = half(W3 x) into d_gate / d_up ([tokens][intermediate] fp16, caller's scratch), then
+ * out[t] = half(W2 . half(clamped_swiglu(gate, up))) -- the stage roundings of the reference's
+ * four launches (three GEMVs and v4_swiglu_clamp_kernel). The reference's memset of the
+ * accumulator is not needed: every element of the `hidden` columns of the output rows is written. */
+int aeon_dense_shared_expert_f16(const void* d_x, int x_stride, int tokens, const void* d_w1,
+                                 const void* d_w3, const void* d_w2, void* d_gate, void* d_up,
+                                 void* d_out, int out_stride, int hidden, int intermediate,
+                                 float swiglu_limit, void* stream);
+
 /* moe_router_kernel launch (src/architecture/deepseek_v4/kernels/moe_router.hpp:104-189; host
  * twin cpu_moe_router :29-100): score = f(logit); choice = score + bias (bias added after the
  * activation, nullable); ids = top_k by descending choice, ties to the lowest index; weights =
@@ -266,6 +291,18 @@ typedef struct {
     const float* d_router_bias;   /* fp32 [experts], nullable */
     const aeon_a64_expert* d_experts;
     int scale_group; /* columns per scale of every expert in the table: 128 (0 reads as 128) or 32 */
+    /* The real model's dense fp16 pieces (all optional, NULL = absent):
+     * the router gate as the checkpoint stores it, fp16 [experts][hidden], read by
+     * aeon_moe_layer_decode when d_router_weight is NULL -- logits are then rounded to fp16 and
+     * widened, as dispatch_router does (layer/v4_layer_body_moe.hpp:135-142); and the shared
+     * expert's three row-major fp16 matrices (w1, w3 [intermediate][hidden], w2
+     * [hidden][intermediate]; run_layer_body_moe_shared_expert, :216-256). With has_shared == 0
+     * and the three given, the step writes the shared expert's fp16 output into the output rows
+     * first and the routed sum is added to it -- the reference's order. */
+    const void* d_router_weight_f16;
+    const void* d_shared_w1_f16;
+    const void* d_shared_w3_f16;
+    const void* d_shared_w2_f16;
 } aeon_moe_layer;
 
 size_t aeon_moe_layer_workspace_bytes(const aeon_moe_layer* layer, int max_tokens);
@@ -292,7 +329,8 @@ int aeon_moe_layer_routed(const aeon_moe_layer* layer, const void* d_x, int x_st
 #define AEON_STAGE_GATE_UP 2
 #define AEON_STAGE_DOWN 4
 #define AEON_STAGE_REDUCE 8
-#define AEON_STAGE_ALL 15
+#define AEON_STAGE_DENSE_SHARED 16 /* the dense fp16 shared expert, when the layer has one */
+#define AEON_STAGE_ALL 31
 int aeon_moe_layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int x_stride,
                                  int tokens, const int32_t* d_topk_ids,
                                  const float* d_topk_weights, void* d_out, int out_stride,

@@ -363,6 +363,38 @@ void orc_expert_ffn(const uint32_t* w1p, const uint16_t* w1s,
     if (!hidden_out) free(hidden);
 }
 
+/* dsv4_oracle.hpp:1708-1753 (dense_ffn): the shared expert, an unquantised FFN with row-major
+ * [out][in] weights, the same clamped SwiGLU, no rounding between the stages. w1, w3 are
+ * [intermediate][hidden], w2 [hidden][intermediate], x [tokens][hidden]. `round_stages` != 0 is
+ * the device's view of the same FFN (layer/v4_layer_body_moe.hpp:216-256: gate, up and the
+ * activation are each stored as fp16 before the next stage reads them). */
+void orc_dense_ffn(size_t intermediate, size_t hidden, const double* x, size_t tokens,
+                   const double* w1, const double* w3, const double* w2, double limit,
+                   int clamp_mode, int round_stages, double* hidden_out, double* out) {
+    double* gate = (double*)malloc(intermediate * sizeof(double));
+    double* up = (double*)malloc(intermediate * sizeof(double));
+    double* act = (double*)malloc(intermediate * sizeof(double));
+    for (size_t t = 0; t < tokens; ++t) {
+        orc_matvec(intermediate, hidden, w1, x + t * hidden, gate);
+        orc_matvec(intermediate, hidden, w3, x + t * hidden, up);
+        for (size_t i = 0; i < intermediate; ++i) {
+            double g = gate[i], u = up[i];
+            if (round_stages) {
+                g = orc_half_bits_to_double(orc_double_to_half_bits(g));
+                u = orc_half_bits_to_double(orc_double_to_half_bits(u));
+            }
+            double h = orc_clamped_swiglu(g, u, limit, clamp_mode);
+            if (round_stages) h = orc_half_bits_to_double(orc_double_to_half_bits(h));
+            act[i] = h;
+            if (hidden_out) hidden_out[t * intermediate + i] = h;
+        }
+        orc_matvec(hidden, intermediate, w2, act, out + t * hidden);
+    }
+    free(gate);
+    free(up);
+    free(act);
+}
+
 /* ------------------------------------------------------------------------------------ */
 /* router                                                                                */
 /* ------------------------------------------------------------------------------------ */

@@ -105,6 +105,9 @@ void orc_expert_ffn(const uint32_t* w1p, const uint16_t* w1s,
 void orc_topk_indices(const double* scores, size_t n, size_t k, int32_t* ids);
 /* dsv4_oracle.hpp:1186-1223. score_kind 0 = sqrt(softplus) (:1168-1176), 1 = sigmoid
  * (:485-487). bias may be NULL. weights[k] = unbiased score / sum * scaling. */
+void orc_dense_ffn(size_t intermediate, size_t hidden, const double* x, size_t tokens,
+                   const double* w1, const double* w3, const double* w2, double limit,
+                   int clamp_mode, int round_stages, double* hidden_out, double* out);
 void orc_router_scores(const double* logits, size_t n, int score_kind, double* scores);
 void orc_router_topk(const double* logits, const double* bias, size_t experts,
                      size_t top_k, double scaling, int score_kind,

@@ -244,6 +244,24 @@ def expert_ffn(w1, w3, w2, H, I, x, limit, clamp_mode=0, round_hidden=False, cfg
     return (out, hidden) if want_hidden else out
 
 
+def dense_ffn(w1, w3, w2, x, limit, clamp_mode=0, round_stages=False, want_hidden=False):
+    """The unquantised shared expert: w1, w3 [I][H], w2 [H][I] (row-major), x [tokens][H]."""
+    w1, w3, w2 = (np.ascontiguousarray(w, dtype=np.float64) for w in (w1, w3, w2))
+    I, H = w1.shape
+    x2 = np.ascontiguousarray(np.atleast_2d(x), dtype=np.float64)
+    t = x2.shape[0]
+    out = np.empty((t, H), dtype=np.float64)
+    hidden = np.empty((t, I), dtype=np.float64) if want_hidden else None
+    lib().orc_dense_ffn(C.c_size_t(I), C.c_size_t(H), _ptr(x2, C.c_double), C.c_size_t(t),
+                        _ptr(w1, C.c_double), _ptr(w3, C.c_double), _ptr(w2, C.c_double),
+                        C.c_double(limit), int(clamp_mode), int(round_stages),
+                        _ptr(hidden, C.c_double), _ptr(out, C.c_double))
+    if np.ndim(x) == 1:
+        out = out[0]
+        hidden = hidden[0] if hidden is not None else None
+    return (out, hidden) if want_hidden else out
+
+
 def topk_indices(scores, k):
     s = np.ascontiguousarray(scores, dtype=np.float64)
     ids = np.empty(min(k, s.size), dtype=np.int32)

@@ -107,6 +107,19 @@ void ref_expert_ffn(const uint8_t* payload, const double* activation, double lim
     std::memcpy(out, r.data(), r.size() * sizeof(double));
 }
 
+void ref_dense_ffn(size_t intermediate, size_t hidden, const double* x, const double* w1,
+                   const double* w3, const double* w2, double limit, int mode, double* out) {
+    const std::vector<double> r = ref::dense_ffn(
+        intermediate, hidden, std::vector<double>(x, x + hidden),
+        std::vector<double>(w1, w1 + intermediate * hidden),
+        std::vector<double>(w3, w3 + intermediate * hidden),
+        std::vector<double>(w2, w2 + hidden * intermediate), limit,
+        mode == 0 ? ref::ClampMode::Asymmetric
+        : mode == 1 ? ref::ClampMode::Symmetric
+                    : ref::ClampMode::None);
+    std::memcpy(out, r.data(), r.size() * sizeof(double));
+}
+
 void ref_topk_indices(const double* scores, size_t n, size_t k, int32_t* ids) {
     const std::vector<int32_t> r = ref::topk_indices(std::vector<double>(scores, scores + n), k);
     std::memcpy(ids, r.data(), r.size() * sizeof(int32_t));

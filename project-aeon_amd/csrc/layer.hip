@@ -14,6 +14,14 @@ extern "C" size_t aeon_router_logits_workspace_bytes(int tokens, int hidden, int
 
 namespace aeon355 {
 
+// csrc/dense.hip
+int launch_dense_gemv(const void* d_x, long x_stride, const void* d_w, void* d_y, long y_stride,
+                      float* d_y32, int tokens, int in_dim, int out_dim, hipStream_t stream);
+int launch_dense_shared_expert(const void* d_x, long x_stride, int tokens, const void* d_w1,
+                               const void* d_w3, const void* d_w2, void* d_gate, void* d_up,
+                               void* d_out, long out_stride, int hidden, int intermediate, float limit,
+                               hipStream_t stream);
+
 // Up to this many tokens a step is a decode batch; above it, a prefill chunk.
 constexpr int kDecodeMaxTokens = 128;
 // Up to this many tokens the expert kernels read the top-k ids directly (no permutation).
@@ -34,6 +42,8 @@ struct LayerWorkspace {
     int32_t* seg_total;
     uint16_t* hidden;
     float* contrib;
+    uint16_t* dense_gate;   // [tokens][intermediate] fp16 each, for a dense shared expert
+    uint16_t* dense_up;
     int positions;
     int seg_capacity;
     size_t bytes;
@@ -66,6 +76,10 @@ static LayerWorkspace carve(const aeon_moe_layer& L, int tokens, void* base) {
     w.seg_total = reinterpret_cast<int32_t*>(take(sizeof(int32_t)));
     w.hidden = reinterpret_cast<uint16_t*>(take(sizeof(uint16_t) * w.positions * L.intermediate));
     w.contrib = reinterpret_cast<float*>(take(sizeof(float) * static_cast<size_t>(w.positions) * L.hidden));
+    const bool dense_shared = L.d_shared_w1_f16 != nullptr;
+    const size_t dense_bytes = dense_shared ? sizeof(uint16_t) * static_cast<size_t>(tokens) * L.intermediate : 0;
+    w.dense_gate = reinterpret_cast<uint16_t*>(take(dense_bytes));
+    w.dense_up = reinterpret_cast<uint16_t*>(take(dense_bytes));
     w.bytes = at;
     return w;
 }
@@ -81,6 +95,11 @@ static int check_layer(const aeon_moe_layer* L, const char* who) {
                  AEON_ERR_INVALID_ARGUMENT, "%s: bad expert geometry (experts=%d top_k=%d)", who,
                  L->experts, L->top_k);
     AEON_REQUIRE(L->d_experts != nullptr, AEON_ERR_INVALID_ARGUMENT, "%s: null expert table", who);
+    const int dense_given = (L->d_shared_w1_f16 != nullptr) + (L->d_shared_w3_f16 != nullptr) +
+                            (L->d_shared_w2_f16 != nullptr);
+    AEON_REQUIRE(dense_given == 0 || (dense_given == 3 && !L->has_shared), AEON_ERR_INVALID_ARGUMENT,
+                 "%s: a dense shared expert needs all three matrices and has_shared == 0 (the int4 "
+                 "always-on expert and the dense one exclude each other)", who);
     AEON_REQUIRE(L->scale_group == 0 || L->scale_group == 128 || L->scale_group == 32,
                  AEON_ERR_INVALID_ARGUMENT, "%s: scale_group must be 128 (or 0) or 32, not %d", who,
                  L->scale_group);
@@ -197,6 +216,19 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     // concentrates its choices that outweighs the saved launch from three tokens on (measured),
     // so the limit is two.
     const bool slots_direct = tokens <= kSlotTokens;
+    if ((stage_mask & AEON_STAGE_DENSE_SHARED) && layer->d_shared_w1_f16 != nullptr) {
+        // the dense shared expert goes first and writes the output rows; the reduce at the end
+        // takes them as each token's fp16 starting value
+        AEON_REQUIRE(out_stride % 4 == 0, AEON_ERR_INVALID_ARGUMENT,
+                     "%s: the dense shared expert stores 8 bytes at a time (out_stride=%d)", who, out_stride);
+        if (int rc = launch_dense_shared_expert(d_x, x_stride, tokens, layer->d_shared_w1_f16,
+                                                layer->d_shared_w3_f16, layer->d_shared_w2_f16,
+                                                w.dense_gate, w.dense_up, d_out, out_stride,
+                                                layer->hidden, layer->intermediate,
+                                                layer->swiglu_limit, s)) {
+            return rc;
+        }
+    }
     if ((stage_mask & AEON_STAGE_PERMUTATION) && !slots_direct) {
         if (int rc = launch_permutation(p, s)) return rc;
     }
@@ -273,8 +305,8 @@ extern "C" int aeon_moe_layer_decode(const aeon_moe_layer* layer, const void* d_
                                      size_t workspace_bytes, void* stream) {
     const char* who = "aeon_moe_layer_decode";
     if (int rc = check_layer(layer, who)) return rc;
-    AEON_REQUIRE(layer->d_router_weight != nullptr, AEON_ERR_INVALID_ARGUMENT,
-                 "%s: the layer has no router weight", who);
+    AEON_REQUIRE(layer->d_router_weight != nullptr || layer->d_router_weight_f16 != nullptr,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: the layer has no router weight", who);
     AEON_REQUIRE(d_x && d_out && d_topk_ids && d_topk_weights && d_workspace,
                  AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
     AEON_REQUIRE(tokens >= 0 && x_stride >= layer->hidden, AEON_ERR_INVALID_ARGUMENT,
@@ -290,11 +322,23 @@ extern "C" int aeon_moe_layer_decode(const aeon_moe_layer* layer, const void* d_
                      layer->score_kind == AEON_ROUTER_SCORE_SIGMOID,
                  AEON_ERR_INVALID_ARGUMENT, "%s: unknown score kind %d", who, layer->score_kind);
     hipStream_t s = as_stream(stream);
-    if (int rc = launch_router_partials(d_x, x_stride, layer->d_router_weight, w.logits_partial,
-                                        tokens, layer->hidden, layer->experts, s)) {
+    const bool f16_gate = layer->d_router_weight == nullptr;
+    if (f16_gate) {
+        // fp16 gate [experts][hidden]: logits rounded to fp16 and widened; the fp16 copy sits in
+        // the space the fp32 gate's partial sums would take (at least as large)
+        AEON_REQUIRE(layer->experts % 16 == 0 && x_stride % 8 == 0, AEON_ERR_INVALID_ARGUMENT,
+                     "%s: the fp16 gate needs experts %% 16 == 0 and x_stride %% 8 == 0", who);
+        if (int rc = launch_dense_gemv(d_x, x_stride, layer->d_router_weight_f16, w.logits_partial,
+                                       layer->experts, w.logits, tokens, layer->hidden,
+                                       layer->experts, s)) {
+            return rc;
+        }
+    } else if (int rc = launch_router_partials(d_x, x_stride, layer->d_router_weight, w.logits_partial,
+                                               tokens, layer->hidden, layer->experts, s)) {
         return rc;
     }
-    if (int rc = launch_router_topk(w.logits_partial, router_logits_chunks(tokens, layer->hidden),
+    if (int rc = launch_router_topk(f16_gate ? nullptr : w.logits_partial,
+                                    router_logits_chunks(tokens, layer->hidden),
                                     w.logits, layer->d_router_bias, nullptr, nullptr,
                                     d_topk_weights, d_topk_ids, tokens, layer->experts,
                                     layer->top_k, layer->routed_scaling_factor, layer->renormalize,

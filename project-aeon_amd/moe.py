@@ -22,7 +22,9 @@ class MoeLayerStruct(C.Structure):
                 ("score_kind", C.c_int), ("routed_scaling_factor", C.c_float),
                 ("renormalize", C.c_int), ("d_router_weight", C.c_void_p),
                 ("d_router_bias", C.c_void_p), ("d_experts", C.c_void_p),
-                ("scale_group", C.c_int)]
+                ("scale_group", C.c_int), ("d_router_weight_f16", C.c_void_p),
+                ("d_shared_w1_f16", C.c_void_p), ("d_shared_w3_f16", C.c_void_p),
+                ("d_shared_w2_f16", C.c_void_p)]
 
 
 def stream_ptr():
@@ -113,16 +115,26 @@ class MoeLayer:
     the pool's last slot)."""
 
     def __init__(self, pool, experts, top_k, has_shared, swiglu_limit, router_weight=None,
-                 router_bias=None, score_kind=1, routed_scaling_factor=1.0, renormalize=True):
+                 router_bias=None, score_kind=1, routed_scaling_factor=1.0, renormalize=True,
+                 router_weight_f16=None, dense_shared=None):
+        """router_weight: fp32 [hidden][experts]; router_weight_f16: the checkpoint's form, fp16
+        [experts][hidden] (one of the two for decode()). dense_shared: (w1, w3, w2) fp16
+        row-major device tensors of an unquantised shared expert (then has_shared is False)."""
         assert pool.slots == experts + (1 if has_shared else 0)
+        assert dense_shared is None or not has_shared
         self.pool = pool
         self.router_weight = router_weight
+        self.router_weight_f16 = router_weight_f16
+        self.dense_shared = dense_shared
         self.router_bias = router_bias
         self.cfg = MoeLayerStruct(pool.H, pool.I, experts, top_k, int(has_shared), swiglu_limit,
                                   score_kind, routed_scaling_factor, int(renormalize),
                                   router_weight.data_ptr() if router_weight is not None else None,
                                   router_bias.data_ptr() if router_bias is not None else None,
-                                  pool.table.data_ptr(), pool.scale_group)
+                                  pool.table.data_ptr(), pool.scale_group,
+                                  router_weight_f16.data_ptr() if router_weight_f16 is not None else None,
+                                  *[(t.data_ptr() if dense_shared is not None else None)
+                                    for t in (dense_shared or (None, None, None))])
         self.workspace = None
         self.workspace_tokens = 0
 
@@ -134,9 +146,10 @@ class MoeLayer:
         return self.workspace
 
     def _new_out(self, x):
-        # with an always-on expert every output row is overwritten; without one the routed sum
-        # is added to the row, which therefore has to start at zero
-        return torch.empty_like(x) if self.cfg.has_shared else torch.zeros_like(x)
+        # with an always-on expert (int4 or dense) every output row is overwritten; without one
+        # the routed sum is added to the row, which therefore has to start at zero
+        overwritten = self.cfg.has_shared or self.dense_shared is not None
+        return torch.empty_like(x) if overwritten else torch.zeros_like(x)
 
     def decode(self, x, out=None, ids=None, weights=None):
         """x fp16 [tokens][hidden] -> (out fp16 [tokens][hidden], ids int32, weights fp32).
@@ -172,6 +185,12 @@ class MoeLayer:
         tokens = x.shape[0]
         E = self.cfg.experts
         lib = capi.lib()
+        if self.router_weight is None:
+            half = torch.empty(tokens, E, dtype=torch.float16, device=x.device)
+            out = torch.empty(tokens, E, dtype=torch.float32, device=x.device)
+            capi.call("aeon_router_logits_f16", capi.vp(x), x.stride(0), capi.vp(self.router_weight_f16),
+                      capi.vp(half), capi.vp(out), tokens, self.cfg.hidden, E, stream_ptr())
+            return out
         n = lib.aeon_router_logits_workspace_bytes(tokens, self.cfg.hidden, E)
         ws = torch.empty(max(n, 4), dtype=torch.uint8, device=x.device)
         out = torch.empty(tokens, E, dtype=torch.float32, device=x.device)

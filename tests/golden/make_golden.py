@@ -120,6 +120,20 @@ def main():
                  ("norm_out", nout), ("norm_unit", nunit)):
         out["dyn_" + k] = v
 
+    # dense (unquantised) FFN, the shared expert (dsv4_oracle.hpp:1708-1753); its own generator so
+    # the vectors above keep their values
+    drng = np.random.default_rng(77)
+    DI, DH = 48, 80
+    dw1, dw3, dw2 = drng.normal(0, 0.3, (DI, DH)), drng.normal(0, 0.3, (DI, DH)), drng.normal(0, 0.3, (DH, DI))
+    dx = drng.normal(size=DH)
+    for key, limit, mode in (("dense_out_limit10", 10.0, 0), ("dense_out_limit0p25", 0.25, 0),
+                             ("dense_out_symmetric0p25", 0.25, 1)):
+        dy = np.empty(DH)
+        ref.ref_dense_ffn(C.c_size_t(DI), C.c_size_t(DH), P(dx, C.c_double), P(dw1, C.c_double),
+                          P(dw3, C.c_double), P(dw2, C.c_double), C.c_double(limit), mode, P(dy, C.c_double))
+        out[key] = dy
+    out["dense_w1"], out["dense_w3"], out["dense_w2"], out["dense_x"] = dw1, dw3, dw2, dx
+
     path = os.path.join(ROOT, "tests", "golden", "ref_vectors.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path), "bytes")

@@ -68,3 +68,12 @@ def test_swiglu_router_hc(orc, gold):
     assert np.array_equal(orc.hc_mixes(gold["dyn_mix_res"], gold["dyn_mix_fn"]), gold["dyn_mix_out"])
     assert np.array_equal(orc.rmsnorm(gold["dyn_norm_x"], gold["dyn_norm_w"]), gold["dyn_norm_out"])
     assert np.array_equal(orc.rmsnorm(gold["dyn_norm_x"]), gold["dyn_norm_unit"])
+
+
+def test_dense_ffn(orc, gold):
+    for key, limit, mode in (("dense_out_limit10", 10.0, 0), ("dense_out_limit0p25", 0.25, 0),
+                             ("dense_out_symmetric0p25", 0.25, 1)):
+        got = orc.dense_ffn(gold["dense_w1"], gold["dense_w3"], gold["dense_w2"], gold["dense_x"], limit,
+                            clamp_mode=mode)
+        assert np.array_equal(got, gold[key])
+    assert not np.array_equal(gold["dense_out_limit0p25"], gold["dense_out_symmetric0p25"])

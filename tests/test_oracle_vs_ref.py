@@ -167,6 +167,32 @@ def test_expert_ffn_bit_identical_to_reference(orc, ref, mode, limit):
     assert np.abs(want).max() > 1e-3
 
 
+@pytest.mark.parametrize("mode,limit", [(0, 10.0), (0, 0.25), (1, 0.25), (2, 10.0)])
+def test_dense_ffn_bit_identical_to_reference(orc, ref, mode, limit):
+    """dense_ffn (dsv4_oracle.hpp:1708-1753), the unquantised shared expert: same bits, and the
+    closed form of tests/test_v4_shared_expert_oracle.cpp:180-194 (w1 = w3 = w2 = e_0, x0 = 0.5
+    gives silu(0.5) * 0.5 in out[0] and zeros elsewhere)."""
+    rng = np.random.default_rng(8)
+    I, H = 96, 160
+    w1, w3 = rng.normal(0, 0.2, (I, H)), rng.normal(0, 0.2, (I, H))
+    w2 = rng.normal(0, 0.2, (H, I))
+    x = rng.normal(size=H)
+    want = np.empty(H)
+    ref.ref_dense_ffn(C.c_size_t(I), C.c_size_t(H), P(x, C.c_double), P(w1, C.c_double),
+                      P(w3, C.c_double), P(w2, C.c_double), C.c_double(limit), mode,
+                      P(want, C.c_double))
+    got = orc.dense_ffn(w1, w3, w2, x, limit, clamp_mode=mode)
+    assert np.array_equal(got, want)
+    assert np.abs(want).max() > 1e-3
+    e1, e3, e2 = np.zeros((2, 3)), np.zeros((2, 3)), np.zeros((3, 2))
+    e1[0, 0] = e3[0, 0] = e2[0, 0] = 1.0
+    out = orc.dense_ffn(e1, e3, e2, np.array([0.5, 0.0, 0.0]), 10.0)
+    assert abs(out[0] - (0.5 / (1.0 + np.exp(-0.5))) * 0.5) < 1e-15 and out[1] == 0.0 and out[2] == 0.0
+    # the device's view rounds gate, up and the activation to fp16: a different, nearby result
+    rounded = orc.dense_ffn(w1, w3, w2, x, limit, clamp_mode=mode, round_stages=True)
+    assert 0 < np.abs(rounded - got).max() <= 2e-2 * np.abs(got).max()
+
+
 def test_topk_and_router_match_reference(orc, ref):
     rng = np.random.default_rng(6)
     for trial in range(50):
