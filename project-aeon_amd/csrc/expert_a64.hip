@@ -630,16 +630,40 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
     }
 
     // the lane holds tokens 16*mt + 4*chunk..+3 of output row (tile, n)
+    if (GATE_UP) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                store_hidden(gu, acc[0][r][mt], acc[NM - 1][r][mt], first, mt * kSegTokens + chunk * 4, count,
+                             (tile0 + r) * 16 + n);
+            }
+        return;
+    }
+    // Down: the fp32 contributions are the launch's largest output, and four tokens of one row
+    // per lane would be four 4-byte stores each behind its own index and weight load. Every
+    // 16 x 16 result tile is turned round through this wave's quarter of the (now idle)
+    // activation buffer, so that a lane holds four consecutive rows of one token: one index,
+    // one weight, one 16-byte store.
+    float* turn = reinterpret_cast<float*>(xs) + wave * 1024;
+    const bool unit_weight = slot_mode && s == seg.slot_shared;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
+        const int token = mt * kSegTokens + n;
+        const bool live = token < count;
+        const int position = first + (live ? token : 0);
+        const float w = unit_weight ? 1.0f : dn.weight[position];
+        const size_t out_row = dn.out_row != nullptr ? dn.out_row[position] : position;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int row = (tile0 + r) * 16 + n;
-            if (GATE_UP) {
-                store_hidden(gu, acc[0][r][mt], acc[NM - 1][r][mt], first, mt * kSegTokens + chunk * 4, count, row);
-            } else {
-                store_contrib(dn, acc[0][r][mt], first, mt * kSegTokens + chunk * 4, count, row,
-                              slot_mode && s == seg.slot_shared);
+            float* tile = turn + ((mt * R + r) & 3) * 256;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) tile[(chunk * 4 + v) * 16 + n] = acc[0][r][mt][v];
+            __builtin_amdgcn_wave_barrier();
+            const float4_t rows = *reinterpret_cast<const float4_t*>(tile + n * 16 + chunk * 4);
+            if (live) {
+                const float4_t value = {w * rows[0], w * rows[1], w * rows[2], w * rows[3]};
+                *reinterpret_cast<float4_t*>(dn.contrib + out_row * dn.H + (tile0 + r) * 16 + chunk * 4) = value;
             }
         }
     }

@@ -16,6 +16,7 @@
 //     than two token tiles of padding.
 // Weights are read once per (expert, position tile); tiles of one expert are adjacent in the
 // grid so their re-reads meet in L2 / Infinity Cache.
+#include <cstdlib>
 #include <type_traits>
 
 #include "expert_a64.hpp"
@@ -60,7 +61,7 @@ __device__ __forceinline__ half8_t scaled_fragment(uint32_t word, half2_t scale2
 template <bool GATE_UP, int R, int LIVE, int DEPTH, int SG>
 __device__ __forceinline__ void grouped_run(const SegGateUpArgs& gu, const SegDownArgs& dn,
                                                  const aeon_a64_expert& e, int first, int count,
-                                                 half8_t* xs_flat) {
+                                                 half8_t* xs_flat, int nblock) {
     static_assert(LIVE >= 1 && LIVE <= kGroupedMT, "a window holds at most kGroupedMT token tiles");
     constexpr int NM = GATE_UP ? 2 : 1;
     constexpr int STAGES = DEPTH + 1;
@@ -76,7 +77,7 @@ __device__ __forceinline__ void grouped_run(const SegGateUpArgs& gu, const SegDo
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: LDS-DMA targets stay scalar
     const int n = lane & 15;
     const int chunk = lane >> 4;
-    const int tile0 = (blockIdx.x * 4 + wave) * R;
+    const int tile0 = (nblock * 4 + wave) * R;
 
     const int K = GATE_UP ? gu.H : dn.I;
     const int groups = K / 128;
@@ -290,7 +291,14 @@ template <bool GATE_UP, int R, int SG>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void a64_grouped_kernel(
     SegGateUpArgs gu, SegDownArgs dn) {
     const SegmentList& seg = GATE_UP ? gu.seg : dn.seg;
-    const int s = blockIdx.y;
+    int s = blockIdx.y;
+    int nblock = blockIdx.x;
+    if ((GATE_UP ? gu.grid_map : dn.grid_map) == 1) {
+        const int linear = blockIdx.y * gridDim.x + blockIdx.x;
+        const int slot = linear >> 3;
+        s = (slot / gridDim.x) * 8 + (linear & 7);
+        nblock = slot % gridDim.x;
+    }
     if (s >= *seg.total) return;
     const int first = seg.first[s];
     const int count = seg.count[s];
@@ -303,18 +311,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     const int live_tiles = (count + 15) >> 4;
     if (live_tiles > 6) {
-        grouped_run<GATE_UP, R, 8, 1, SG>(gu, dn, e, first, count, xs);
+        grouped_run<GATE_UP, R, 8, 1, SG>(gu, dn, e, first, count, xs, nblock);
     } else if (live_tiles > 4) {
-        grouped_run<GATE_UP, R, 6, 1, SG>(gu, dn, e, first, count, xs);
+        grouped_run<GATE_UP, R, 6, 1, SG>(gu, dn, e, first, count, xs, nblock);
     } else if (live_tiles > 3) {
-        grouped_run<GATE_UP, R, 4, 3, SG>(gu, dn, e, first, count, xs);
+        grouped_run<GATE_UP, R, 4, 3, SG>(gu, dn, e, first, count, xs, nblock);
     } else if (live_tiles > 2) {
-        grouped_run<GATE_UP, R, 3, 3, SG>(gu, dn, e, first, count, xs);
+        grouped_run<GATE_UP, R, 3, 3, SG>(gu, dn, e, first, count, xs, nblock);
     } else if (live_tiles > 1) {
-        grouped_run<GATE_UP, R, 2, 3, SG>(gu, dn, e, first, count, xs);
+        grouped_run<GATE_UP, R, 2, 3, SG>(gu, dn, e, first, count, xs, nblock);
     } else {
-        grouped_run<GATE_UP, R, 1, 3, SG>(gu, dn, e, first, count, xs);
+        grouped_run<GATE_UP, R, 1, 3, SG>(gu, dn, e, first, count, xs, nblock);
     }
+}
+
+static int grouped_grid_map() {
+    static const int v = [] { const char* e = getenv("AEON_GROUPED_MAP"); return e ? atoi(e) : 0; }();
+    return v;
 }
 
 int launch_grouped_gate_up(const SegGateUpArgs& a, hipStream_t stream) {
@@ -326,10 +339,13 @@ int launch_grouped_gate_up(const SegGateUpArgs& a, hipStream_t stream) {
     if (a.seg.capacity <= 0) return AEON_OK;
     AEON_REQUIRE(a.scales_per_group == 1 || a.scales_per_group == 4, AEON_ERR_INVALID_ARGUMENT,
                  "grouped gate/up: %d scales per 128 columns (1 or 4)", a.scales_per_group);
+    SegGateUpArgs b = a;
+    b.grid_map = grouped_grid_map();
+    const int cap = (a.seg.capacity + 7) & ~7;
     if (a.scales_per_group == 4) {
-        a64_grouped_kernel<true, 2, 4><<<dim3(a.I / 128, a.seg.capacity), 256, 0, stream>>>(a, SegDownArgs{});
+        a64_grouped_kernel<true, 2, 4><<<dim3(a.I / 128, cap), 256, 0, stream>>>(b, SegDownArgs{});
     } else {
-        a64_grouped_kernel<true, 2, 1><<<dim3(a.I / 128, a.seg.capacity), 256, 0, stream>>>(a, SegDownArgs{});
+        a64_grouped_kernel<true, 2, 1><<<dim3(a.I / 128, cap), 256, 0, stream>>>(b, SegDownArgs{});
     }
     AEON_LAUNCH_CHECK();
     return AEON_OK;
@@ -343,10 +359,13 @@ int launch_grouped_down(const SegDownArgs& a, hipStream_t stream) {
     if (a.seg.capacity <= 0) return AEON_OK;
     AEON_REQUIRE(a.scales_per_group == 1 || a.scales_per_group == 4, AEON_ERR_INVALID_ARGUMENT,
                  "grouped down: %d scales per 128 columns (1 or 4)", a.scales_per_group);
+    SegDownArgs b = a;
+    b.grid_map = grouped_grid_map();
+    const int cap = (a.seg.capacity + 7) & ~7;
     if (a.scales_per_group == 4) {
-        a64_grouped_kernel<false, 4, 4><<<dim3(a.H / 256, a.seg.capacity), 256, 0, stream>>>(SegGateUpArgs{}, a);
+        a64_grouped_kernel<false, 4, 4><<<dim3(a.H / 256, cap), 256, 0, stream>>>(SegGateUpArgs{}, b);
     } else {
-        a64_grouped_kernel<false, 4, 1><<<dim3(a.H / 256, a.seg.capacity), 256, 0, stream>>>(SegGateUpArgs{}, a);
+        a64_grouped_kernel<false, 4, 1><<<dim3(a.H / 256, cap), 256, 0, stream>>>(SegGateUpArgs{}, b);
     }
     AEON_LAUNCH_CHECK();
     return AEON_OK;
