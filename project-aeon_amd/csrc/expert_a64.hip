@@ -45,14 +45,18 @@ struct GemvArgs {
     int scales_per_group;  // 1 (one fp16 per row and 128 columns) or 4 (one per 32 columns)
 };
 
-template <int NMAT, int TOK, int WK, int SG>
+// HALF: a workgroup takes 8 of a tile's 16 rows (the lanes of the other 8 stay idle), so that a
+// matrix with fewer than 256 row tiles still puts a workgroup on every CU: such a launch is a
+// few microseconds long and bound by latency, not by the bytes a wave moves.
+template <int NMAT, int TOK, int WK, int SG, bool HALF>
 __global__ __launch_bounds__(WK * 64) void a64_gemv_kernel(GemvArgs a) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int r = lane & 15;
     const int chunk = lane >> 4;
-    const int tile = blockIdx.x;
+    const int tile = HALF ? blockIdx.x >> 1 : blockIdx.x;
     const size_t tile_base = static_cast<size_t>(tile) * a.groups;
+    const bool mine = !HALF || (r >> 3) == static_cast<int>(blockIdx.x & 1);
 
     float acc[NMAT][TOK];
 #pragma unroll
@@ -71,7 +75,7 @@ __global__ __launch_bounds__(WK * 64) void a64_gemv_kernel(GemvArgs a) {
 #pragma unroll
         for (int j = 0; j < kGemvPrefetch; ++j) {
             const int g = g0 + j * WK;
-            if (g < a.groups) {
+            if (g < a.groups && mine) {
                 wq[0][j] = a.pa[(tile_base + g) * 64 + lane];
                 sc[0][j] = load_scale(a.sa, g);
                 if (NMAT == 2) {
@@ -83,7 +87,7 @@ __global__ __launch_bounds__(WK * 64) void a64_gemv_kernel(GemvArgs a) {
 #pragma unroll
         for (int j = 0; j < kGemvPrefetch; ++j) {
             const int g = g0 + j * WK;
-            if (g < a.groups) {
+            if (g < a.groups && mine) {
 #pragma unroll
                 for (int t = 0; t < TOK; ++t) {
                     if (t < a.tokens) {
@@ -134,7 +138,7 @@ __global__ __launch_bounds__(WK * 64) void a64_gemv_kernel(GemvArgs a) {
         const int row = i & 15;
         const int t = (i >> 4) % TOK;
         const int m = (i >> 4) / TOK;
-        if (t < a.tokens) {
+        if (t < a.tokens && (!HALF || (row >> 3) == static_cast<int>(blockIdx.x & 1))) {
             float sum = 0.0f;
 #pragma unroll
             for (int w = 0; w < WK; ++w) sum += partial[w][m][t][row];
@@ -158,13 +162,15 @@ __global__ __launch_bounds__(WK * 64) void a64_gemv_kernel(GemvArgs a) {
 
 template <int NMAT, int TOK, int SG>
 static int launch_gemv_wk_sg(const GemvArgs& a, int wk, hipStream_t stream) {
-    const dim3 grid(a.N / 16);
-    if (wk >= 16) {
-        a64_gemv_kernel<NMAT, TOK, 16, SG><<<grid, 16 * 64, 0, stream>>>(a);
+    const int tiles = a.N / 16;
+    if (wk >= 16 && tiles < 256) {
+        a64_gemv_kernel<NMAT, TOK, 16, SG, true><<<dim3(2 * tiles), 16 * 64, 0, stream>>>(a);
+    } else if (wk >= 16) {
+        a64_gemv_kernel<NMAT, TOK, 16, SG, false><<<dim3(tiles), 16 * 64, 0, stream>>>(a);
     } else if (wk >= 8) {
-        a64_gemv_kernel<NMAT, TOK, 8, SG><<<grid, 8 * 64, 0, stream>>>(a);
+        a64_gemv_kernel<NMAT, TOK, 8, SG, false><<<dim3(tiles), 8 * 64, 0, stream>>>(a);
     } else {
-        a64_gemv_kernel<NMAT, TOK, 4, SG><<<grid, 4 * 64, 0, stream>>>(a);
+        a64_gemv_kernel<NMAT, TOK, 4, SG, false><<<dim3(tiles), 4 * 64, 0, stream>>>(a);
     }
     AEON_LAUNCH_CHECK();
     return AEON_OK;
