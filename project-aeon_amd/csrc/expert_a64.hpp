@@ -44,7 +44,6 @@ struct SegGateUpArgs {
     aeon_a64_expert direct_expert;
     int direct_count;
     int scales_per_group;     // 1: one fp16 scale per (row, 128 columns); 4: one per 32 columns
-    int grid_map;
 };
 
 struct SegDownArgs {
@@ -63,7 +62,6 @@ struct SegDownArgs {
     uint16_t* fused_out;
     const uint16_t* fused_initial;
     int scales_per_group;     // as in SegGateUpArgs
-    int grid_map;
 };
 
 // k_split: 1, 2 or 4 waves of a workgroup split K between them; 0 = the wide form (four waves,

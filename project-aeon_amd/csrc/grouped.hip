@@ -16,7 +16,6 @@
 //     than two token tiles of padding.
 // Weights are read once per (expert, position tile); tiles of one expert are adjacent in the
 // grid so their re-reads meet in L2 / Infinity Cache.
-#include <cstdlib>
 #include <type_traits>
 
 #include "expert_a64.hpp"
@@ -291,14 +290,14 @@ template <bool GATE_UP, int R, int SG>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void a64_grouped_kernel(
     SegGateUpArgs gu, SegDownArgs dn) {
     const SegmentList& seg = GATE_UP ? gu.seg : dn.seg;
-    int s = blockIdx.y;
-    int nblock = blockIdx.x;
-    if ((GATE_UP ? gu.grid_map : dn.grid_map) == 1) {
-        const int linear = blockIdx.y * gridDim.x + blockIdx.x;
-        const int slot = linear >> 3;
-        s = (slot / gridDim.x) * 8 + (linear & 7);
-        nblock = slot % gridDim.x;
-    }
+    // Workgroups go to the eight XCDs round robin by their linear index, and every XCD has an L2
+    // of its own. Index i therefore serves window 8*(i/8/blocks) + i%8, row block (i/8)%blocks:
+    // all row blocks of one window run on one XCD and fetch the window's activations into that
+    // L2 once, not once per XCD.
+    const int linear = blockIdx.y * gridDim.x + blockIdx.x;
+    const int slot = linear >> 3;
+    const int s = (slot / gridDim.x) * 8 + (linear & 7);
+    const int nblock = slot % gridDim.x;
     if (s >= *seg.total) return;
     const int first = seg.first[s];
     const int count = seg.count[s];
@@ -325,11 +324,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
-static int grouped_grid_map() {
-    static const int v = [] { const char* e = getenv("AEON_GROUPED_MAP"); return e ? atoi(e) : 0; }();
-    return v;
-}
-
 int launch_grouped_gate_up(const SegGateUpArgs& a, hipStream_t stream) {
     AEON_REQUIRE(a.H % 128 == 0 && a.I % 128 == 0 && a.x_stride % 8 == 0, AEON_ERR_INVALID_ARGUMENT,
                  "grouped gate/up: need H%%128==0, I%%128==0 and an activation pitch that keeps "
@@ -339,13 +333,11 @@ int launch_grouped_gate_up(const SegGateUpArgs& a, hipStream_t stream) {
     if (a.seg.capacity <= 0) return AEON_OK;
     AEON_REQUIRE(a.scales_per_group == 1 || a.scales_per_group == 4, AEON_ERR_INVALID_ARGUMENT,
                  "grouped gate/up: %d scales per 128 columns (1 or 4)", a.scales_per_group);
-    SegGateUpArgs b = a;
-    b.grid_map = grouped_grid_map();
-    const int cap = (a.seg.capacity + 7) & ~7;
+    const int cap = (a.seg.capacity + 7) & ~7;   // whole rounds of the eight XCDs
     if (a.scales_per_group == 4) {
-        a64_grouped_kernel<true, 2, 4><<<dim3(a.I / 128, cap), 256, 0, stream>>>(b, SegDownArgs{});
+        a64_grouped_kernel<true, 2, 4><<<dim3(a.I / 128, cap), 256, 0, stream>>>(a, SegDownArgs{});
     } else {
-        a64_grouped_kernel<true, 2, 1><<<dim3(a.I / 128, cap), 256, 0, stream>>>(b, SegDownArgs{});
+        a64_grouped_kernel<true, 2, 1><<<dim3(a.I / 128, cap), 256, 0, stream>>>(a, SegDownArgs{});
     }
     AEON_LAUNCH_CHECK();
     return AEON_OK;
@@ -359,13 +351,11 @@ int launch_grouped_down(const SegDownArgs& a, hipStream_t stream) {
     if (a.seg.capacity <= 0) return AEON_OK;
     AEON_REQUIRE(a.scales_per_group == 1 || a.scales_per_group == 4, AEON_ERR_INVALID_ARGUMENT,
                  "grouped down: %d scales per 128 columns (1 or 4)", a.scales_per_group);
-    SegDownArgs b = a;
-    b.grid_map = grouped_grid_map();
     const int cap = (a.seg.capacity + 7) & ~7;
     if (a.scales_per_group == 4) {
-        a64_grouped_kernel<false, 4, 4><<<dim3(a.H / 256, cap), 256, 0, stream>>>(SegGateUpArgs{}, b);
+        a64_grouped_kernel<false, 4, 4><<<dim3(a.H / 256, cap), 256, 0, stream>>>(SegGateUpArgs{}, a);
     } else {
-        a64_grouped_kernel<false, 4, 1><<<dim3(a.H / 256, cap), 256, 0, stream>>>(SegGateUpArgs{}, b);
+        a64_grouped_kernel<false, 4, 1><<<dim3(a.H / 256, cap), 256, 0, stream>>>(SegGateUpArgs{}, a);
     }
     AEON_LAUNCH_CHECK();
     return AEON_OK;
