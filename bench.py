@@ -253,17 +253,42 @@ def run_dropin(capi, moe, torch, np):
     torch.cuda.synchronize()
     del experts
     res["resident"] = []
-    for T, live in ((1, 64), (8, 64), (64, 64), (256, 64), (1024, 64), (256, 256)):
+    # the reference's recorded routing: the layer-0 prefill histogram of its first real prompt
+    # (the distribution tests/bench_expert_pair_ab.cpp:189-262 draws its chunks from: six
+    # distinct experts per token by rejection, weights 0.55/(slot+1)+0.03)
+    profile = os.path.join(ROOT, "tests", "golden", "routing_first_real_prompt_layer0.csv")
+    counts = np.loadtxt(profile, delimiter=",", skiprows=1)[:, 1]
+    cumulative = np.cumsum(counts / counts.sum())
+
+    def recorded_ids(tokens, rng):
+        ids = np.empty((tokens, K), dtype=np.int32)
+        for t in range(tokens):
+            chosen = []
+            while len(chosen) < K:
+                e = min(int(np.searchsorted(cumulative, rng.random(), side="left")), NE - 1)
+                if e not in chosen:
+                    chosen.append(e)
+            ids[t] = chosen
+        return ids
+
+    cases = [(T, live, "uniform") for T, live in ((1, 64), (8, 64), (64, 64), (256, 64), (1024, 64), (256, 256))]
+    cases += [(T, 256, "recorded") for T in (16, 64, 256, 1024)]
+    for T, live, routing in cases:
         layer = moe.MoeLayer(pool, NE, K, False, limit)
         rng = np.random.default_rng(T)
         rot = []
         for r in range(8):
-            if T == 1:
+            if routing == "recorded":
+                ids_h = recorded_ids(T, rng)
+            elif T == 1:
                 ids_h = np.array([[(K * (r + 1) + j) % live for j in range(K)]], dtype=np.int32)
             else:
                 ids_h = np.stack([rng.permutation(live)[:K] for _ in range(T)]).astype(np.int32)
             rot.append(torch.from_numpy(ids_h).cuda())
-        w = torch.full((T, K), 1.0 / K, device="cuda")
+        if routing == "recorded":
+            w = (0.55 / (torch.arange(K, device="cuda") + 1.0) + 0.03).repeat(T, 1).contiguous()
+        else:
+            w = torch.full((T, K), 1.0 / K, device="cuda")
         xin = (torch.rand(T, H, device="cuda") - 0.5).half()
         outb = torch.zeros(T, H, dtype=torch.float16, device="cuda")
 
@@ -279,7 +304,8 @@ def run_dropin(capi, moe, torch, np):
         torch.cuda.synchronize()
         ms = a.elapsed_time(b) / reps
         touched = np.mean([len(np.unique(r.cpu().numpy())) for r in rot])
-        res["resident"].append({"tokens": T, "experts_live": live, "distinct_experts": round(float(touched), 1),
+        res["resident"].append({"tokens": T, "routing": routing, "experts_live": live,
+                                "distinct_experts": round(float(touched), 1),
                                 "ms": round(ms, 4), "us_per_token": round(ms * 1e3 / T, 2),
                                 "weights_gbps": round(touched * expert_bytes / ms / 1e6, 1),
                                 "tflops": round(2.0 * T * K * 3 * H * I / ms / 1e9, 1)})
