@@ -67,6 +67,29 @@ def settle(fn, torch, seconds=0.3):
         torch.cuda.synchronize()
 
 
+def calibrate_read(capi, torch):
+    """What a read-only stream sustains from HBM on this GPU: 1.5 GiB (the size of a decode
+    step's gate/up weights at batch 64) read once by 1024..12288 workgroups."""
+    nbytes = 3 << 29
+    buf = torch.randint(0, 2 ** 31 - 1, (nbytes // 4,), dtype=torch.int32, device="cuda")
+    out = {"bytes": nbytes, "hbm_peak_gbps": HBM_PEAK_GBPS}
+    for wgs in (1024, 2048, 3072, 4096, 6144, 12288):
+        sink = torch.empty(wgs * 256, dtype=torch.int32, device="cuda")
+
+        def launch(i=0):
+            capi.call("aeon_calibrate_read_stream", capi.vp(buf), C.c_size_t(nbytes), wgs,
+                      capi.vp(sink), C.c_size_t(sink.numel()), None)
+        settle(launch, torch, seconds=0.3)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(20):
+            launch()
+        b.record()
+        torch.cuda.synchronize()
+        out["read_gbps_%d_workgroups" % wgs] = round(nbytes * 20 / (a.elapsed_time(b) * 1e-3) / 1e9, 1)
+    return out
+
+
 def calibrate_mfma(capi, torch):
     """Sustained fp16 matrix-pipe rates of this GPU, for reading the prefill figure: the
     library's register-resident MFMA loop (two waves per SIMD) with constant and with random
@@ -89,6 +112,24 @@ def calibrate_mfma(capi, torch):
         b.record()
         torch.cuda.synchronize()
         out["mfma_loop_tflops_" + name] = round(flop.value * 5 / (a.elapsed_time(b) * 1e-3) / 1e12, 1)
+    # the same loop with the grouped GEMM's companion instructions between the MFMAs
+    mix = {}
+    for valu, lds in ((0, 0), (1, 0), (2, 0), (3, 0), (4, 0), (1, 4), (2, 4), (3, 4), (1, 8), (3, 8)):
+        flop = C.c_double(0.0)
+
+        def launch(i=0):
+            capi.call("aeon_calibrate_mfma_mix", valu, lds, 20000, wgs, capi.vp(sink),
+                      C.c_size_t(sink.numel()), C.byref(flop), None)
+        settle(launch, torch, seconds=0.3)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(5):
+            launch()
+        b.record()
+        torch.cuda.synchronize()
+        mix["%d_valu_%d_lds_reads_per_16" % (valu, lds)] = round(
+            flop.value * 5 / (a.elapsed_time(b) * 1e-3) / 1e12, 1)
+    out["mfma_mix_tflops_random_operands"] = mix
     n = 8192
     x = torch.randn(n, n, device="cuda", dtype=torch.float16)
     y = torch.randn(n, n, device="cuda", dtype=torch.float16)
@@ -547,6 +588,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only copy 1 GiB device to device a few times and exit: the known-size kernel "
                          "the FETCH_SIZE / WRITE_SIZE counters are scaled by")
+    ap.add_argument("--calibrate-read", action="store_true",
+                    help="time a read-only stream over 1.5 GiB and exit")
     ap.add_argument("--calibrate-mfma", action="store_true",
                     help="only measure the sustained fp16 MFMA rate (register-resident loop with "
                          "constant and with random operands) and a library fp16 GEMM, for context")
@@ -596,6 +639,9 @@ def main():
         return
     if args.calibrate_mfma:
         print(json.dumps(calibrate_mfma(capi, torch)))
+        return
+    if args.calibrate_read:
+        print(json.dumps(calibrate_read(capi, torch)))
         return
     if args.dropin:
         print(json.dumps({"dropin": run_dropin(capi, moe, torch, np)}))

@@ -493,6 +493,23 @@ int aeon_synth_matrix_swizzled(uint64_t seed, int expert, int matrix, int N, int
 int aeon_calibrate_mfma_f16(int random_operands, int iterations, int workgroups, float* d_sink,
                             size_t sink_floats, double* flop, void* stream);
 
+/* The same loop with random operands and, after every MFMA, `valu_per_mfma` independent VALU
+ * instructions of the int4 unpack (v_and_or_b32, v_pk_add_f16), plus `lds_reads_per_16` 16-byte
+ * LDS reads per 16 MFMAs. Served pairs: (0..4, 0), (1..3, 4), (1, 8), (3, 8); any other pair is an
+ * AEON_ERR_INVALID_ARGUMENT. Gives the rate an instruction mix reaches with no memory wait at
+ * all, which is what the grouped GEMM's window bodies are read against. */
+int aeon_calibrate_mfma_mix(int valu_per_mfma, int lds_reads_per_16, int iterations,
+                            int workgroups, float* d_sink, size_t sink_floats, double* flop,
+                            void* stream);
+
+/* Launches `workgroups` workgroups that each read their own contiguous bytes/workgroups share
+ * of d_buffer once (16-byte loads, eight in flight per lane; the share must be a multiple of
+ * 32 KiB) and write one folded word per thread to d_sink (>= workgroups*256 words). Timed by
+ * the caller, it gives the rate a read-only stream sustains from HBM on this GPU: the practical
+ * ceiling of the weight-streaming kernels next to the published bandwidth. */
+int aeon_calibrate_read_stream(const void* d_buffer, size_t bytes, int workgroups,
+                               uint32_t* d_sink, size_t sink_words, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

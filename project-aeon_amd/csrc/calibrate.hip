@@ -1,4 +1,4 @@
-// Measurement aid: the rate at which this GPU sustains v_mfma_f32_16x16x32_f16 out of registers,
+// Measurement aids. First: the rate at which this GPU sustains v_mfma_f32_16x16x32_f16 out of registers,
 // with nothing else running. The sustained clock under dense MFMA work depends on the operand
 // data (constant operands toggle few wires; random ones draw more power and clock lower), so the
 // rate with random operands is the practical ceiling the grouped GEMM is read against, beside
@@ -45,9 +45,100 @@ __global__ __launch_bounds__(256) void calibrate_mfma_kernel(float* sink, int it
     sink[blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
+// Third aid: the same MFMA loop with the grouped GEMM's companions issued between the matrix
+// instructions: VALU independent int4-unpack-style VALU instructions after every MFMA and LDS
+// 16-byte LDS reads per 16 MFMAs. MFMA and VALU leave through one issue port per SIMD, so three
+// VALU instructions fill the 16 cycles an MFMA occupies the matrix pipe; the rate measured here
+// is what an instruction mix can reach before any memory wait.
+template <int VALU, int LDS>
+__global__ __launch_bounds__(256) void calibrate_mix_kernel(float* sink, int iterations) {
+    __shared__ u32x4_t lds[256 * 4];
+    half8_t a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t r = calibrate_hash(threadIdx.x * 64 + i * 8 + j + blockIdx.x * 7919);
+            a[i][j] = static_cast<half_t>((static_cast<int>(r & 0xffff) - 32768) / 4096.0f);
+            b[i][j] = static_cast<half_t>((static_cast<int>(r >> 16) - 32768) / 16384.0f);
+        }
+    for (int i = 0; i < 4; ++i) lds[threadIdx.x * 4 + i] = u32x4_t{calibrate_hash(threadIdx.x + i), 1u, 2u, 3u};
+    __syncthreads();
+    float4_t acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    uint32_t x[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = calibrate_hash(threadIdx.x * 8 + i);
+    const uint32_t mask = 0x000f000f, magic = 0x64006400, minus = 0xe408e408;
+    u32x4_t fold = {0u, 0u, 0u, 0u};
+    for (int it = 0; it < iterations; ++it) {
+#pragma unroll
+        for (int m = 0; m < 16; ++m) {
+            // volatile: the order written here is the order issued
+            asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc[m]) : "v"(a[m % 4]), "v"(b[m / 4]));
+#pragma unroll
+            for (int k = 0; k < VALU; ++k) {
+                if (k & 1) asm volatile("v_pk_add_f16 %0, %0, %1" : "+v"(x[(m * VALU + k) % 8]) : "v"(minus));
+                else asm volatile("v_and_or_b32 %0, %0, %1, %2" : "+v"(x[(m * VALU + k) % 8]) : "v"(mask), "v"(magic));
+            }
+            if (LDS > 0 && m % (16 / (LDS > 0 ? LDS : 1)) == 0) {
+                u32x4_t t;
+                asm volatile("ds_read_b128 %0, %1" : "=v"(t) : "v"(static_cast<uint32_t>(threadIdx.x * 16 + (m & 3) * 4096)));
+                fold ^= t;
+            }
+        }
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+    uint32_t bits = fold[0];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) bits ^= x[i];
+    sink[blockIdx.x * blockDim.x + threadIdx.x] = s + static_cast<float>(bits & 1u);
+}
+
+// Second aid: what a read-only stream sustains from HBM. Workgroup w reads its own contiguous
+// share of the buffer, 16 bytes a lane and eight loads in flight per lane (each wave instruction
+// one contiguous KiB, as a weight tile is), folds everything into one word per lane so the loads
+// cannot be dropped, and writes nothing else.
+__global__ __launch_bounds__(256) void calibrate_read_kernel(const u32x4_t* __restrict__ buf,
+                                                             size_t units_per_workgroup,
+                                                             uint32_t* sink) {
+    const u32x4_t* mine = buf + blockIdx.x * units_per_workgroup + threadIdx.x;
+    u32x4_t fold = {0u, 0u, 0u, 0u};
+    for (size_t i = 0; i < units_per_workgroup; i += 8 * 256) {
+        u32x4_t v[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) v[q] = __builtin_nontemporal_load(mine + i + q * 256);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) fold ^= v[q];
+    }
+    sink[blockIdx.x * 256 + threadIdx.x] = fold[0] ^ fold[1] ^ fold[2] ^ fold[3];
+}
+
 }  // namespace aeon355
 
 using namespace aeon355;
+
+extern "C" int aeon_calibrate_read_stream(const void* d_buffer, size_t bytes, int workgroups,
+                                          uint32_t* d_sink, size_t sink_words, void* stream) {
+    const char* who = "aeon_calibrate_read_stream";
+    AEON_REQUIRE(d_buffer != nullptr && d_sink != nullptr && workgroups > 0, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: bad arguments (workgroups=%d)", who, workgroups);
+    const size_t per_workgroup = bytes / static_cast<size_t>(workgroups);
+    AEON_REQUIRE(per_workgroup > 0 && per_workgroup % (8 * 256 * 16) == 0 &&
+                     per_workgroup * workgroups == bytes,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: %zu bytes over %d workgroups is not a whole number "
+                 "of 32 KiB rounds each", who, bytes, workgroups);
+    AEON_REQUIRE(sink_words >= static_cast<size_t>(workgroups) * 256, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: the sink holds %zu words, %zu needed", who, sink_words,
+                 static_cast<size_t>(workgroups) * 256);
+    calibrate_read_kernel<<<workgroups, 256, 0, as_stream(stream)>>>(
+        static_cast<const u32x4_t*>(d_buffer), per_workgroup / 16, d_sink);
+    AEON_LAUNCH_CHECK();
+    return AEON_OK;
+}
 
 extern "C" int aeon_calibrate_mfma_f16(int random_operands, int iterations, int workgroups,
                                        float* d_sink, size_t sink_floats, double* flop,
@@ -65,6 +156,34 @@ extern "C" int aeon_calibrate_mfma_f16(int random_operands, int iterations, int 
     }
     AEON_LAUNCH_CHECK();
     // 4 waves a workgroup, 16 MFMAs a round, 2*16*16*32 FLOP an MFMA
+    if (flop != nullptr) *flop = static_cast<double>(workgroups) * 4.0 * iterations * 16.0 * 16384.0;
+    return AEON_OK;
+}
+
+extern "C" int aeon_calibrate_mfma_mix(int valu_per_mfma, int lds_reads_per_16, int iterations,
+                                       int workgroups, float* d_sink, size_t sink_floats,
+                                       double* flop, void* stream) {
+    const char* who = "aeon_calibrate_mfma_mix";
+    AEON_REQUIRE(d_sink != nullptr && iterations > 0 && workgroups > 0, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: bad arguments (iterations=%d workgroups=%d)", who, iterations, workgroups);
+    AEON_REQUIRE(sink_floats >= static_cast<size_t>(workgroups) * 256, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: the sink holds %zu floats, %zu needed", who, sink_floats,
+                 static_cast<size_t>(workgroups) * 256);
+    hipStream_t s = as_stream(stream);
+    const int key = valu_per_mfma * 100 + lds_reads_per_16;
+#define AEON_MIX_CASE(v_, l_)                                                                   \
+    case (v_) * 100 + (l_):                                                                     \
+        calibrate_mix_kernel<v_, l_><<<workgroups, 256, 0, s>>>(d_sink, iterations);            \
+        break;
+    switch (key) {
+        AEON_MIX_CASE(0, 0) AEON_MIX_CASE(1, 0) AEON_MIX_CASE(2, 0) AEON_MIX_CASE(3, 0) AEON_MIX_CASE(4, 0)
+        AEON_MIX_CASE(1, 4) AEON_MIX_CASE(2, 4) AEON_MIX_CASE(3, 4) AEON_MIX_CASE(1, 8) AEON_MIX_CASE(3, 8)
+        default:
+            AEON_REQUIRE(false, AEON_ERR_INVALID_ARGUMENT, "%s: no kernel for %d VALU per MFMA and %d "
+                         "LDS reads per 16", who, valu_per_mfma, lds_reads_per_16);
+    }
+#undef AEON_MIX_CASE
+    AEON_LAUNCH_CHECK();
     if (flop != nullptr) *flop = static_cast<double>(workgroups) * 4.0 * iterations * 16.0 * 16384.0;
     return AEON_OK;
 }
