@@ -381,6 +381,50 @@ def run_chunk_sweep(layer, moe, synth, torch, np, H, I, E, K_TOP, SEED):
     return rows
 
 
+def run_window_classes(layer, moe, capi, synth, torch, np, H, I, E, K_TOP, SEED):
+    """The grouped (prefill) kernels under routings that isolate one window size each: every
+    routed expert gets exactly n positions (tokens = n * experts / top_k; the always-on expert's
+    tokens fill whole windows of their own), n from 8 to 512. Gate/up and down are timed alone by
+    stage mask; `us_per_window` divides the gate/up launch by its number of windows. Chunks of at
+    most 128 tokens would take the decode kernels, so n starts where the grouped ones do."""
+    rows = []
+    for n in (8, 16, 32, 48, 64, 96, 128, 256, 512):
+        T = n * E // K_TOP
+        ids_h = ((np.arange(T)[:, None] * K_TOP + np.arange(K_TOP)[None, :]) % E).astype(np.int32)
+        ids = torch.from_numpy(ids_h).cuda()
+        w = torch.full((T, K_TOP), 1.0 / K_TOP, dtype=torch.float32, device="cuda")
+        x = torch.from_numpy(synth.activations(SEED, T, H, unit=3)).cuda()
+        out = torch.empty(T, H, dtype=torch.float16, device="cuda")
+        ws = layer._workspace(T)
+
+        def stages(mask):
+            capi.call("aeon_moe_layer_routed_stages", C.byref(layer.cfg), capi.vp(x), x.stride(0), T,
+                      capi.vp(ids), capi.vp(w), capi.vp(out), out.stride(0), capi.vp(ws),
+                      C.c_size_t(ws.numel()), mask, moe.stream_ptr())
+
+        def timed(mask):
+            settle(lambda i: stages(mask), torch, 0.2)
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(10):
+                stages(mask)
+            b.record()
+            torch.cuda.synchronize()
+            return a.elapsed_time(b) / 10
+
+        stages(15)
+        gu, dn, al = timed(2), timed(4), timed(15)
+        positions = T * K_TOP + T
+        flop = 2.0 * positions * H * I
+        windows = E * ((n + 127) // 128) + (T + 127) // 128
+        rows.append({"positions_per_expert": n, "tokens": T, "windows": windows,
+                     "step_ms": round(al, 3), "step_tflops": round(3 * flop / al / 1e9, 1),
+                     "gate_up_ms": round(gu, 3), "gate_up_tflops": round(2 * flop / gu / 1e9, 1),
+                     "gate_up_us_per_window": round(gu * 1e3 / windows, 2),
+                     "down_ms": round(dn, 3), "down_tflops": round(flop / dn / 1e9, 1)})
+    return rows
+
+
 def run_prefill(layer, moe, capi, synth, torch, np, H, I, E, K_TOP, SEED, steps, warmup):
     """BASELINE config 3: 2048 tokens, top-8 of 256 experts with Zipf(1.1) popularity, through the
     permutation -> grouped gate+up GEMM + SwiGLU -> grouped W2 GEMM -> fixed-order reduce path.
@@ -596,6 +640,9 @@ def main():
     ap.add_argument("--dropin", action="store_true",
                     help="only time the entry points that read the .aeon layout in place, at the "
                          "reference's own shape (hidden 4096, top-6, one scale per 32 columns)")
+    ap.add_argument("--window-classes", action="store_true",
+                    help="also time the grouped kernels with every expert holding the same number "
+                         "of positions (8..512), into `window_classes`")
     ap.add_argument("--chunk-sweep", action="store_true",
                     help="also time the routed step at 64..1024 tokens (uniform and Zipf routing) "
                          "into `chunk_sweep`")
@@ -875,6 +922,9 @@ def main():
         result["prefill"] = prefill
     if sweep is not None:
         result["sweep"] = sweep
+    if args.window_classes:
+        result["window_classes"] = run_window_classes(layer, moe, capi, synth, torch, np, H, I, E,
+                                                      K_TOP, SEED)
     if args.chunk_sweep:
         result["chunk_sweep"] = run_chunk_sweep(layer, moe, synth, torch, np, H, I, E, K_TOP, SEED)
     print(json.dumps(result))
