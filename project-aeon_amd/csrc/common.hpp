@@ -66,6 +66,36 @@ __device__ __forceinline__ const AEON_GLOBAL T* as_global(const void* p) {
     return (const AEON_GLOBAL T*)(p);
 }
 
+// A decode launch reads every weight once, while activations, scales (whose cache lines are
+// shared between neighbouring row tiles), tables and expert lists are read again and again by
+// other workgroups. The streaming ("non-temporal") hint on the weight loads keeps them from
+// pushing the re-read data out of the caches: measured on the batch-64 decode step, 0.412 ->
+// 0.371 ms with nothing else changed (with the hint on the scales as well: 0.375). Where
+// weights ARE read again -- the prefill windows of a hot expert -- the hint costs (2.27 -> 2.39
+// ms), so the grouped kernels load normally.
+template <class T>
+__device__ __forceinline__ T stream_load(const T* p) {
+    return __builtin_nontemporal_load(p);
+}
+template <class T>
+__device__ __forceinline__ T stream_load(const AEON_GLOBAL T* p) {
+    return __builtin_nontemporal_load(p);
+}
+__device__ __forceinline__ uint4 stream_load(const uint4* p) {
+    const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ uint2 stream_load(const uint2* p) {
+    const u32x2_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(p));
+    return make_uint2(v[0], v[1]);
+}
+
+template <bool STREAM, class P>
+__device__ __forceinline__ auto load_maybe_stream(P p) {
+    if constexpr (STREAM) return stream_load(p);
+    else return *p;
+}
+
 union Word2Half {
     uint32_t u;
     half2_t h;

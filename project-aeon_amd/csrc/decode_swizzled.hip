@@ -105,16 +105,20 @@ __global__ __launch_bounds__(kWaves * 64) void swizzled_decode_kernel(SwzArgs a)
     const size_t block_base = static_cast<size_t>(row_block) * a.iterations * 32 + lane32;
     uint4 wa[kMaxSteps], wb[kMaxSteps];
     uint16_t ca[kMaxSteps], cb[kMaxSteps];
+    // The expert-table modes stream several experts' weights per launch past the activation
+    // rows they share: there the streaming hint pays (26.5 -> 25.4 us for the per-token trio).
+    // The single-matrix launches are one trip to memory long and 0.5-1 us slower with it.
+    constexpr bool kStream = !(MODE == SwzMode::Gemv || MODE == SwzMode::Dual);
     auto fetch = [&](int first_step) {
 #pragma unroll
         for (int j = 0; j < kMaxSteps; ++j) {
             const int it = 2 * (first_step + j) + half_id;
             const size_t slot = block_base + static_cast<size_t>(it < a.iterations ? it : a.iterations - 1) * 32;
-            wa[j] = pa[slot];
-            ca[j] = sa[slot];
+            wa[j] = load_maybe_stream<kStream>(&pa[slot]);
+            ca[j] = load_maybe_stream<kStream>(&sa[slot]);
             if (kTwo) {
-                wb[j] = pb[slot];
-                cb[j] = sb[slot];
+                wb[j] = load_maybe_stream<kStream>(&pb[slot]);
+                cb[j] = load_maybe_stream<kStream>(&sb[slot]);
             }
         }
     };

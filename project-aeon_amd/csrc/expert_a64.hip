@@ -15,6 +15,7 @@
 //     in fp32 to the per-group MFMA result, so dequantisation stays exact.
 #include "expert_a64.hpp"
 
+
 namespace aeon355 {
 
 // ---------------------------------------------------------------------------------------------
@@ -76,10 +77,10 @@ __global__ __launch_bounds__(WK * 64) void a64_gemv_kernel(GemvArgs a) {
         for (int j = 0; j < kGemvPrefetch; ++j) {
             const int g = g0 + j * WK;
             if (g < a.groups && mine) {
-                wq[0][j] = a.pa[(tile_base + g) * 64 + lane];
+                wq[0][j] = stream_load(&a.pa[(tile_base + g) * 64 + lane]);
                 sc[0][j] = load_scale(a.sa, g);
                 if (NMAT == 2) {
-                    wq[1][j] = a.pb[(tile_base + g) * 64 + lane];
+                    wq[1][j] = stream_load(&a.pb[(tile_base + g) * 64 + lane]);
                     sc[1][j] = load_scale(a.sb, g);
                 }
             }
@@ -366,7 +367,7 @@ __global__ __launch_bounds__(WK * 64) void a64_seg_kernel(SegGateUpArgs gu, SegD
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 const size_t t = static_cast<size_t>(tile0 + r) * groups + g;
-                wq[d][m][r] = pm[m][t * 64 + lane];
+                wq[d][m][r] = stream_load(&pm[m][t * 64 + lane]);
                 sc[d][m][r].load(sm[m] + t * (16 * SG), n);
             }
 #pragma unroll
@@ -539,7 +540,7 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 const size_t t = static_cast<size_t>(tile0 + r) * groups + g;
-                wq[d][m][r] = pm[m][t * 64 + lane];
+                wq[d][m][r] = stream_load(&pm[m][t * 64 + lane]);
             }
     };
     // LDS image of a group's activations: [buffer][token tile][MFMA step][lane] x 16 bytes
@@ -817,7 +818,7 @@ __global__ __launch_bounds__(256) void token_reduce_kernel(
         for (int q = 0; q < 4; ++q) acc[q] = half_bits_to_float(initial[t * initial_stride + i + q]);
     }
     const float* c = contrib + static_cast<size_t>(t) * slots * hidden + i;
-    // Eight slots at a time: their rows are requested first, whether they count or not (a
+    // The contributions are read once (streaming loads). Eight slots at a time: their rows are requested first, whether they count or not (a
     // dropped slot's row is stale but addressable), so that no request waits for an id; the ids
     // only decide which of the loaded rows are added, in slot order.
     for (int s0 = 0; s0 < slots; s0 += 8) {
@@ -825,7 +826,7 @@ __global__ __launch_bounds__(256) void token_reduce_kernel(
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int s = s0 + j < slots ? s0 + j : slots - 1;
-            v[j] = *reinterpret_cast<const float4_t*>(c + static_cast<size_t>(s) * hidden);
+            v[j] = stream_load(reinterpret_cast<const float4_t*>(c + static_cast<size_t>(s) * hidden));
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j) {

@@ -116,13 +116,18 @@ __device__ __forceinline__ void grouped_swizzled_window(const GroupedSwzArgs& a,
     constexpr int kAhead = MT <= 2 ? kDepth : 1;   // divides kDepth: pass G's slot is G % kAhead
     uint4 wa4[kDepth], wb4[kDepth];
     uint16_t s_a[kDepth], s_b[kDepth];
+    // A window of one or two token tiles mostly belongs to an expert with no other window, whose
+    // weights nobody reads again: streamed past the caches. Larger windows usually have
+    // siblings of the same expert that find the weights in L2, so they load normally (with the
+    // hint on them a 1024-token chunk went from 0.92 to 1.03 ms).
+    constexpr bool kStream = MT <= 2;
     auto fetch_weights = [&](int d, int G) {
         const size_t slot = slot_of(G < passes ? G : passes - 1);
-        wa4[d] = qa[slot];
-        s_a[d] = sa[slot];
+        wa4[d] = load_maybe_stream<kStream>(&qa[slot]);
+        s_a[d] = load_maybe_stream<kStream>(&sa[slot]);
         if (GATE_UP) {
-            wb4[d] = qb[slot];
-            s_b[d] = sb[slot];
+            wb4[d] = load_maybe_stream<kStream>(&qb[slot]);
+            s_b[d] = load_maybe_stream<kStream>(&sb[slot]);
         } else {
             wb4[d] = make_uint4(0, 0, 0, 0);
             s_b[d] = 0;
