@@ -30,6 +30,9 @@ struct SegmentList {
     int slot_shared;
     int slot_top_k;
     int slot_tokens;   // <= kSegTokens
+    // [capacity], optional: nonzero where the segment is its expert's only one, i.e. nobody else
+    // reads that expert's weights in this launch
+    const int* alone = nullptr;
 };
 
 struct SegGateUpArgs {

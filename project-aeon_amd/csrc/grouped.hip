@@ -57,7 +57,7 @@ __device__ __forceinline__ half8_t scaled_fragment(uint32_t word, half2_t scale2
 // Loads complete in issue order and every group issues the same number, so "group g+1 has
 // landed" is a bound on the count of outstanding loads; a group ends in a bare s_barrier (the
 // fences of __syncthreads would wait for every LDS-DMA request and drain the ring).
-template <bool GATE_UP, int R, int LIVE, int DEPTH, int SG>
+template <bool GATE_UP, int R, int LIVE, int DEPTH, int SG, bool STREAM>
 __device__ __forceinline__ void grouped_run(const SegGateUpArgs& gu, const SegDownArgs& dn,
                                                  const aeon_a64_expert& e, int first, int count,
                                                  half8_t* xs_flat, int nblock) {
@@ -137,8 +137,8 @@ __device__ __forceinline__ void grouped_run(const SegGateUpArgs& gu, const SegDo
         }                                                                                           \
         _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                            \
             _Pragma("unroll") for (int r = 0; r < R; ++r) {                                         \
-                wq[stage_][m][r] = *(const AEON_GLOBAL u32x4_t*)(                                   \
-                    pm[m] + (woff[r] + static_cast<uint32_t>(gi_) * 1024u));                        \
+                wq[stage_][m][r] = load_maybe_stream<STREAM>((const AEON_GLOBAL u32x4_t*)(          \
+                    pm[m] + (woff[r] + static_cast<uint32_t>(gi_) * 1024u)));                       \
                 sc[stage_][m][r] = *(const AEON_GLOBAL RowScales*)(                                 \
                     sm[m] + (soff[r] + static_cast<uint32_t>(gi_) * (32u * SG)));                   \
             }                                                                                       \
@@ -308,20 +308,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // window, or a deeper ring of smaller ones.
     __shared__ half8_t xs[2 * kGroupedMT * 4 * 64];
 
+    // A window that is its expert's only one reads weights nobody reads again: streamed past the
+    // caches. The windows of a hot expert find each other's weights in L2 and load normally.
+    const bool alone = seg.alone != nullptr && seg.alone[s] != 0;
     const int live_tiles = (count + 15) >> 4;
+#define AEON_RUN(live_, depth_)                                                                  \
+    do {                                                                                         \
+        if (alone) grouped_run<GATE_UP, R, live_, depth_, SG, true>(gu, dn, e, first, count, xs, nblock);  \
+        else grouped_run<GATE_UP, R, live_, depth_, SG, false>(gu, dn, e, first, count, xs, nblock);       \
+    } while (0)
     if (live_tiles > 6) {
-        grouped_run<GATE_UP, R, 8, 1, SG>(gu, dn, e, first, count, xs, nblock);
+        AEON_RUN(8, 1);
     } else if (live_tiles > 4) {
-        grouped_run<GATE_UP, R, 6, 1, SG>(gu, dn, e, first, count, xs, nblock);
+        AEON_RUN(6, 1);
     } else if (live_tiles > 3) {
-        grouped_run<GATE_UP, R, 4, 3, SG>(gu, dn, e, first, count, xs, nblock);
+        AEON_RUN(4, 3);
     } else if (live_tiles > 2) {
-        grouped_run<GATE_UP, R, 3, 3, SG>(gu, dn, e, first, count, xs, nblock);
+        AEON_RUN(3, 3);
     } else if (live_tiles > 1) {
-        grouped_run<GATE_UP, R, 2, 3, SG>(gu, dn, e, first, count, xs, nblock);
+        AEON_RUN(2, 3);
     } else {
-        grouped_run<GATE_UP, R, 1, 3, SG>(gu, dn, e, first, count, xs, nblock);
+        AEON_RUN(1, 3);
     }
+#undef AEON_RUN
 }
 
 int launch_grouped_gate_up(const SegGateUpArgs& a, hipStream_t stream) {

@@ -40,6 +40,7 @@ struct LayerWorkspace {
     int32_t* seg_first;
     int32_t* seg_count;
     int32_t* seg_total;
+    int32_t* seg_alone;
     uint16_t* hidden;
     float* contrib;
     uint16_t* dense_gate;   // [tokens][intermediate] fp16 each, for a dense shared expert
@@ -74,6 +75,7 @@ static LayerWorkspace carve(const aeon_moe_layer& L, int tokens, void* base) {
     w.seg_first = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * w.seg_capacity));
     w.seg_count = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * w.seg_capacity));
     w.seg_total = reinterpret_cast<int32_t*>(take(sizeof(int32_t)));
+    w.seg_alone = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * w.seg_capacity));
     w.hidden = reinterpret_cast<uint16_t*>(take(sizeof(uint16_t) * w.positions * L.intermediate));
     w.contrib = reinterpret_cast<float*>(take(sizeof(float) * static_cast<size_t>(w.positions) * L.hidden));
     const bool dense_shared = L.d_shared_w1_f16 != nullptr;
@@ -164,6 +166,7 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     p.seg_first = w.seg_first;
     p.seg_count = w.seg_count;
     p.seg_total = w.seg_total;
+    p.seg_alone = w.seg_alone;
     // A decode batch walks segments of one expert's positions with the weight-streaming kernels;
     // a prefill chunk walks 128-position tiles with the grouped GEMM.
     const bool grouped = tokens > kDecodeMaxTokens;
@@ -238,7 +241,8 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     gu.x_stride = x_stride;
     gu.row_index = w.token_indices;
     gu.experts = layer->d_experts;
-    gu.seg = SegmentList{w.seg_expert, w.seg_first, w.seg_count, w.seg_total, p.seg_capacity, 0, -1, 0, 0};
+    gu.seg = SegmentList{w.seg_expert, w.seg_first, w.seg_count, w.seg_total, p.seg_capacity, 0, -1, 0, 0,
+                         w.seg_alone};
     if (slots_direct) {
         gu.seg = SegmentList{d_topk_ids, nullptr, nullptr, nullptr,
                              draws + (layer->has_shared ? 1 : 0), layer->experts,

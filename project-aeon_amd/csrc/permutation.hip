@@ -117,6 +117,7 @@ __global__ __launch_bounds__(1024) void permutation_offsets_kernel(PermutationAr
                 a.seg_expert[at] = e;
                 a.seg_first[at] = offset + s * a.seg_tokens;
                 a.seg_count[at] = min(a.seg_tokens, count - s * a.seg_tokens);
+                if (a.seg_alone != nullptr) a.seg_alone[at] = segments == 1 ? 1 : 0;
             }
         }
         if (e == 0) *a.seg_total = min(all, a.seg_capacity);

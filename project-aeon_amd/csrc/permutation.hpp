@@ -29,6 +29,7 @@ struct PermutationArgs {
     int32_t* seg_total;
     int seg_tokens;
     int seg_capacity;
+    int32_t* seg_alone = nullptr;  // optional [seg_capacity]: 1 where a list has a single segment
 };
 
 int launch_permutation(const PermutationArgs& a, hipStream_t stream);
