@@ -22,8 +22,15 @@ int launch_dense_shared_expert(const void* d_x, long x_stride, int tokens, const
                                void* d_out, long out_stride, int hidden, int intermediate, float limit,
                                hipStream_t stream);
 
-// Up to this many tokens a step is a decode batch; above it, a prefill chunk.
+// Up to this many tokens a step always runs on the weight-streaming (decode) kernels. Above it
+// the grouped GEMM takes over once the experts hold enough positions each for its windows to
+// fill: more than kGroupedMinPerExpert draws per routed expert on average. Measured (decode
+// kernels against grouped): hidden 7168, top-8 of 256, uniform / Zipf routing: 129 tokens (4 per
+// expert) 0.93 / 0.73 against 1.06 / 0.80 ms; 256 tokens (8) 1.00 / 1.00 against 1.12 / 1.04;
+// 512 tokens (16) 1.22 / 1.40 against 1.28 / 1.31. Hidden 4096, top-6 of 64, 256 tokens (24 per
+// expert): 0.237 against 0.213 ms.
 constexpr int kDecodeMaxTokens = 128;
+constexpr int kGroupedMinPerExpert = 12;
 // Up to this many tokens the expert kernels read the top-k ids directly (no permutation).
 constexpr int kSlotTokens = 2;
 
@@ -169,7 +176,8 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     p.seg_alone = w.seg_alone;
     // A decode batch walks segments of one expert's positions with the weight-streaming kernels;
     // a prefill chunk walks 128-position tiles with the grouped GEMM.
-    const bool grouped = tokens > kDecodeMaxTokens;
+    const bool grouped = tokens > kDecodeMaxTokens &&
+                         static_cast<long>(draws) > static_cast<long>(kGroupedMinPerExpert) * layer->experts;
     const int lists = layer->experts + (layer->has_shared ? 1 : 0);
 
     // Few live segments (a small batch) leave the chip idle unless K is also split.

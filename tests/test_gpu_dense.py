@@ -134,7 +134,7 @@ def test_fp16_gate_logits_and_routing(orc):
         assert 17 not in ids[t] or 5 in ids[t]
 
 
-@pytest.mark.parametrize("T", [1, 9, 64, 200])
+@pytest.mark.parametrize("T", [1, 9, 64, 200, 300])
 def test_layer_step_with_the_checkpoint_pieces(orc, T):
     """The layer step as the real model composes it: fp16 gate, sqrt(softplus) score with bias
     after it, top-6 scaled by 1.5, group-32 int4 routed experts, the dense fp16 shared expert

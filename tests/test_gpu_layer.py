@@ -394,12 +394,14 @@ def test_config2_full_size_sampled(orc):
 
 
 @pytest.mark.parametrize("H,I,B", [(256, 128, 3), (256, 384, 5), (768, 256, 17), (256, 128, 70),
-                                   (256, 128, 128), (256, 128, 129)])
+                                   (256, 128, 128), (256, 128, 129), (256, 128, 256),
+                                   (256, 128, 257)])
 def test_layer_on_minimal_shapes(orc, H, I, B):
     """Shapes with fewer 128-column groups than a workgroup has K-split waves (a wave with no
     group of its own must not fetch anything outside the matrix), odd group counts for the
-    pipeline tails, and batches at and just over the grouped path's threshold (128 tokens) on a
-    one-group K."""
+    pipeline tails, and batches at and just over the grouped path's threshold (128 tokens; with
+    five experts every larger batch has enough positions per expert for it) and around two full
+    windows (256, 257) on a one-group K."""
     torch, h, capi, moe, synth = _setup()
     E, k, limit = 5, 2, 7.0
     pool = moe.ExpertPool(E + 1, H, I)
@@ -417,7 +419,39 @@ def test_layer_on_minimal_shapes(orc, H, I, B):
     assert np.abs(out - want).max() <= 6e-3 * np.abs(want).max()
 
 
-@pytest.mark.parametrize("T", [1, 6, 150])
+@pytest.mark.parametrize("T,E,k", [(300, 64, 2), (200, 256, 4), (383, 128, 4)])
+def test_chunks_with_few_positions_per_expert_stay_on_the_decode_kernels(orc, T, E, k):
+    """Above 128 tokens the grouped GEMM only takes over when the experts hold more than twelve
+    draws each on average; a chunk of many tokens over many experts keeps the weight-streaming
+    kernels (segments of up to 32 positions, several per expert where the routing concentrates).
+    Sampled tokens against the oracle, and the same chunk cut into two calls of at most 128
+    tokens -- which always run on those kernels -- has to give the same bits (a token's result
+    does not depend on which other tokens share its segment; the shapes are such that whole and
+    parts take the same form, K-split or wide, of each launch)."""
+    torch, h, capi, moe, synth = _setup()
+    H, I, limit = 512, 256, 7.0
+    assert T > 128 and T * k <= 12 * E
+    pool = moe.ExpertPool(E + 1, H, I)
+    assert pool.fill_synthetic(seed=71, first_expert_id=0) == 0
+    layer = moe.MoeLayer(pool, E, k, True, limit)
+    ids, w = synth.zipf_routing(71, T, E, k, s=1.1)
+    x = synth.activations(71, T, H)
+    d_x, d_ids, d_w = h.dev_half(x), h.to_dev(ids), h.to_dev(w)
+    out = layer.routed(d_x, d_ids, d_w)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    cut = 128
+    parts = [layer.routed(d_x[a:b].contiguous(), d_ids[a:b].contiguous(), d_w[a:b].contiguous()).cpu().numpy()
+             for a, b in ((0, cut), (cut, min(2 * cut, T)), (min(2 * cut, T), T)) if b > a]
+    assert np.array_equal(np.concatenate(parts), got)
+    rows = sorted(set([0, T // 2, T - 1, 129 % T]))
+    experts = {int(e): h.Expert(71, int(e), H, I) for e in np.unique(ids[rows])}
+    shared = h.Expert(71, E, H, I)
+    want = _oracle_layer(orc, h, experts, x[rows], ids[rows], w[rows], shared, limit)
+    assert np.abs(got[rows] - want).max() <= 6e-3 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("T", [1, 6, 150, 300])
 def test_out_of_range_ids_contribute_nothing(orc, T):
     """An id outside [0, experts) is dropped by the permutation (as the reference's does); the
     slot-ordered reduce must then leave that slot out instead of adding a row nobody wrote. Run
@@ -636,7 +670,7 @@ def test_config3_prefill_full_size_sampled(orc):
 
 def test_random_layer_steps_against_oracle(orc):
     """Forty seeded random layer steps (hidden, intermediate, expert count, top-k, token count
-    from 1 to 200, with and without an always-on expert, two ids out of range each): every token
+    from 1 to 300, with and without an always-on expert, two ids out of range each): every token
     count class of the step -- direct slots, decode segments, grouped windows -- lands here with
     shapes the other tests do not use. Odd cases keep a scale of their own per 32 columns (the
     `.aeon` format's grouping, four scales per 128 columns in the packing), even ones one per
@@ -649,7 +683,7 @@ def test_random_layer_steps_against_oracle(orc):
         I = int(rng.choice([128, 256, 384, 512]))
         E = int(rng.integers(2, 40))
         k = int(rng.integers(1, min(E, 8) + 1))
-        T = int(rng.choice([1, 2, 3, 5, 16, 17, 33, 64, 100, 128, 129, 200]))
+        T = int(rng.choice([1, 2, 3, 5, 16, 17, 33, 64, 100, 128, 129, 200, 257, 300]))
         shared = bool(rng.integers(0, 2))
         seed = 500 + case
         scale_group = 32 if case % 2 else 128
@@ -684,7 +718,7 @@ def test_random_layer_steps_against_oracle(orc):
             assert np.abs(out[t] - want).max() <= 6e-3 * max(np.abs(want).max(), 1e-6), (what, t)
 
 
-@pytest.mark.parametrize("B", [1, 8, 150])
+@pytest.mark.parametrize("B", [1, 8, 150, 300])
 def test_layer_step_replays_from_a_captured_graph(orc, B):
     """The step allocates nothing, clears nothing with a memset and never synchronises, so it can
     be recorded into a HIP graph: the graph is replayed four times with new activations copied
