@@ -384,11 +384,11 @@ def run_chunk_sweep(layer, moe, synth, torch, np, H, I, E, K_TOP, SEED):
 def run_window_classes(layer, moe, capi, synth, torch, np, H, I, E, K_TOP, SEED):
     """The grouped (prefill) kernels under routings that isolate one window size each: every
     routed expert gets exactly n positions (tokens = n * experts / top_k; the always-on expert's
-    tokens fill whole windows of their own), n from 8 to 512. Gate/up and down are timed alone by
-    stage mask; `us_per_window` divides the gate/up launch by its number of windows. Chunks of at
-    most 128 tokens would take the decode kernels, so n starts where the grouped ones do."""
+    tokens fill whole windows of their own), n from 16 to 512. Gate/up and down are timed alone by
+    stage mask; `us_per_window` divides the gate/up launch by its number of windows. Chunks whose
+    experts average twelve draws or fewer take the decode kernels, so n starts above that."""
     rows = []
-    for n in (8, 16, 32, 48, 64, 96, 128, 256, 512):
+    for n in (16, 32, 48, 64, 96, 128, 256, 512):
         T = n * E // K_TOP
         ids_h = ((np.arange(T)[:, None] * K_TOP + np.arange(K_TOP)[None, :]) % E).astype(np.int32)
         ids = torch.from_numpy(ids_h).cuda()
@@ -642,7 +642,7 @@ def main():
                          "reference's own shape (hidden 4096, top-6, one scale per 32 columns)")
     ap.add_argument("--window-classes", action="store_true",
                     help="also time the grouped kernels with every expert holding the same number "
-                         "of positions (8..512), into `window_classes`")
+                         "of positions (16..512), into `window_classes`")
     ap.add_argument("--chunk-sweep", action="store_true",
                     help="also time the routed step at 64..1024 tokens (uniform and Zipf routing) "
                          "into `chunk_sweep`")
