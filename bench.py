@@ -897,7 +897,13 @@ def main():
                      "frac": round(main_run["gate_up_gbps"] / HBM_PEAK_GBPS, 4),
                      "avg_launch_ms": round(main_run["gate_up_ms"], 4),
                      "algorithmic_bytes": int(main_run["gate_up_bytes"]),
-                     "traffic": measured_traffic(B, E, args.router_bias_scale)},
+                     "traffic": measured_traffic(B, E, args.router_bias_scale),
+                     # hardware counters cannot be read from inside this process: the figure is
+                     # the profiler's, taken on this command and kept with its source
+                     "traffic_source": ("profiles/traffic_config2_decode_b%d.json (rocprofv3 --pmc "
+                                        "FETCH_SIZE / WRITE_SIZE per dispatch of this command, scaled "
+                                        "by --calibrate-copy)" % B)
+                     if measured_traffic(B, E, args.router_bias_scale) is not None else None},
         "down_kernel": {"achieved_gbps": round(main_run["down_gbps"], 1),
                         "avg_launch_ms": round(main_run["down_ms"], 4),
                         "algorithmic_bytes": int(main_run["down_bytes"])},
