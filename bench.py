@@ -37,9 +37,13 @@ def _package():
     return sys.modules["project_aeon_amd"]
 
 
+SCALE_GROUP = 128   # columns per fp16 scale in the resident packing (--scale-group)
+
+
 def matrix_bytes(n, k):
-    """Algorithmic bytes of one int4 matrix: packed nibbles + one fp16 scale per 128 columns."""
-    return n * k // 2 + n * (k // 128) * 2
+    """Algorithmic bytes of one int4 matrix: packed nibbles + one fp16 scale per SCALE_GROUP
+    columns (128: config 2 as written; 32: the `.aeon` checkpoint's own grouping)."""
+    return n * k // 2 + n * (k // SCALE_GROUP) * 2
 
 
 def measured_traffic(batch, experts, bias_scale=1.0):
@@ -554,7 +558,7 @@ def run_other_configs(pool, layer, moe, capi, synth, torch, np, H, I, E, K_TOP, 
     # residual streams between layers
     layers, mixes = [layer], []
     for l in range(1, 4):
-        p = moe.ExpertPool(E + 1, H, I)
+        p = moe.ExpertPool(E + 1, H, I, scale_group=SCALE_GROUP)
         assert p.fill_synthetic(seed=SEED + 100 * l, first_expert_id=0) == 0
         wr_l = torch.from_numpy(synth.router_weight(SEED + 100 * l, H, E)).cuda()
         bias_l = torch.from_numpy(synth.router_bias(SEED + 100 * l, E)).cuda()
@@ -640,6 +644,10 @@ def main():
     ap.add_argument("--dropin", action="store_true",
                     help="only time the entry points that read the .aeon layout in place, at the "
                          "reference's own shape (hidden 4096, top-6, one scale per 32 columns)")
+    ap.add_argument("--scale-group", type=int, default=128, choices=(32, 128),
+                    help="columns per fp16 scale of the resident experts in the headline and prefill "
+                         "legs: 128 (config 2 as written) or 32 (the checkpoint format's grouping, "
+                         "four scales kept per 128 columns)")
     ap.add_argument("--window-classes", action="store_true",
                     help="also time the grouped kernels with every expert holding the same number "
                          "of positions (16..512), into `window_classes`")
@@ -697,7 +705,9 @@ def main():
     B = args.batch
 
     t_setup = time.time()
-    pool = moe.ExpertPool(E + 1, H, I)
+    global SCALE_GROUP
+    SCALE_GROUP = args.scale_group
+    pool = moe.ExpertPool(E + 1, H, I, scale_group=SCALE_GROUP)
     bad = pool.fill_synthetic(seed=SEED, first_expert_id=0)
     assert bad == 0, "repack found group-32 scales that differ inside a 128-group"
     wr = torch.from_numpy(synth.router_weight(SEED, H, E)).cuda()
@@ -882,8 +892,8 @@ def main():
         "dtype": "int4 weights x fp16 activations, fp32 accumulate",
         "data": "synthetic (seeded int4 experts generated and re-swizzled on the device)",
         "config": {"workload": "config2: full MoE layer decode, batch %d, hidden 7168, "
-                               "intermediate 2048, top-8 of %d experts + 1 shared, group-128 int4"
-                               % (B, E),
+                               "intermediate 2048, top-8 of %d experts + 1 shared, group-%d int4"
+                               % (B, E, SCALE_GROUP),
                    "router_bias_scale": args.router_bias_scale,
                    "batch": B, "experts": E, "resident_expert_bytes": pool.payload_bytes * (E + 1),
                    "distinct_routed_experts_per_step": round(main_run["distinct_experts_mean"], 1)},
