@@ -468,7 +468,7 @@ bool seg_wide_fits(bool gate_up, int row_tiles, int k_dim, int scales_per_group)
     return kWideActivationLdsBytes + seg_wide_scale_lds_bytes(gate_up, row_tiles, k_dim, scales_per_group) <= 65536;
 }
 
-template <bool GATE_UP, int R, int D, int MT, int SG>
+template <bool GATE_UP, int R, int D, int MT, int SG, bool SL>
 __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const SegDownArgs& dn, int s,
                                               int row_block, half8_t* xs, u32x4_t* scale_lds) {
     constexpr int NM = GATE_UP ? 2 : 1;
@@ -514,16 +514,21 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
         }
     }
 
+    // SL: the scales of this wave's tiles over all of K are copied to LDS once. Otherwise (four
+    // scales per group over a K too long for that) they ride in the register ring with the
+    // weights, fetched from memory a group at a time.
     const int tile_u4 = groups * 2 * SG;    // 32 (SG 1) or 128 (SG 4) bytes of scales per group
     u32x4_t* my_scales = scale_lds + static_cast<size_t>(wave) * NM * R * tile_u4;
+    if constexpr (SL) {
 #pragma unroll
-    for (int m = 0; m < NM; ++m)
+        for (int m = 0; m < NM; ++m)
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const AEON_GLOBAL u32x4_t* src = reinterpret_cast<const AEON_GLOBAL u32x4_t*>(
-                sm[m] + static_cast<size_t>(tile0 + r) * groups * (16 * SG));
-            for (int i = lane; i < tile_u4; i += 64) my_scales[(m * R + r) * tile_u4 + i] = src[i];
-        }
+            for (int r = 0; r < R; ++r) {
+                const AEON_GLOBAL u32x4_t* src = reinterpret_cast<const AEON_GLOBAL u32x4_t*>(
+                    sm[m] + static_cast<size_t>(tile0 + r) * groups * (16 * SG));
+                for (int i = lane; i < tile_u4; i += 64) my_scales[(m * R + r) * tile_u4 + i] = src[i];
+            }
+    }
 
     float4_t acc[NM][R][MT];
 #pragma unroll
@@ -534,6 +539,7 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
             for (int mt = 0; mt < MT; ++mt) acc[m][r][mt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
     u32x4_t wq[D][NM][R];
+    RowScales<SG> ring_scales[SL ? 1 : D][NM][R];
     auto load_group = [&](int d, int g) {
 #pragma unroll
         for (int m = 0; m < NM; ++m)
@@ -541,6 +547,7 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
             for (int r = 0; r < R; ++r) {
                 const size_t t = static_cast<size_t>(tile0 + r) * groups + g;
                 wq[d][m][r] = stream_load(&pm[m][t * 64 + lane]);
+                if constexpr (!SL) ring_scales[d][m][r].load(sm[m] + t * (16 * SG), n);
             }
     };
     // LDS image of a group's activations: [buffer][token tile][MFMA step][lane] x 16 bytes
@@ -583,8 +590,10 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
 #pragma unroll
         for (int m = 0; m < NM; ++m)
 #pragma unroll
-            for (int r = 0; r < R; ++r)
-                sc[m][r].load_lds(scale_halves + ((m * R + r) * tile_u4 + g * 2 * SG) * 8, n);
+            for (int r = 0; r < R; ++r) {
+                if constexpr (SL) sc[m][r].load_lds(scale_halves + ((m * R + r) * tile_u4 + g * 2 * SG) * 8, n);
+                else sc[m][r] = ring_scales[d][m][r];
+            }
         // The K steps run outermost and the wave's tiles innermost, so that consecutive matrix
         // instructions belong to different accumulators: a chain of dependent ones would hold
         // the SIMD for the latency of each.
@@ -679,7 +688,7 @@ __device__ __forceinline__ void seg_wide_item(const SegGateUpArgs& gu, const Seg
 // Four waves per SIMD (128 registers a wave) is what hides the weight stream's latency for the
 // common one-tile segment; the rarer two-tile path is kept inside that budget by a shallower
 // prefetch ring rather than allowed to halve everyone's occupancy.
-template <bool GATE_UP, int R, int D, int SG>
+template <bool GATE_UP, int R, int D, int SG, bool SL>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void a64_seg_wide_kernel(
     SegGateUpArgs gu, SegDownArgs dn) {
     __shared__ half8_t xs[2 * kWideMaxTiles * 4 * 64];
@@ -692,14 +701,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             const int id = seg.expert[s];
             if (id < 0 || id >= seg.slot_experts) return;
         }
-        seg_wide_item<GATE_UP, R, D, 1, SG>(gu, dn, s, blockIdx.x, xs, scale_lds);
+        seg_wide_item<GATE_UP, R, D, 1, SG, SL>(gu, dn, s, blockIdx.x, xs, scale_lds);
         return;
     }
     if (s >= *seg.total) return;
     if (seg.count[s] > kSegTokens) {
-        seg_wide_item<GATE_UP, R, (SG == 4 ? 1 : D > 2 ? 2 : D), 2, SG>(gu, dn, s, blockIdx.x, xs, scale_lds);
+        seg_wide_item<GATE_UP, R, (SG == 4 ? 1 : D > 2 ? 2 : D), 2, SG, SL>(gu, dn, s, blockIdx.x, xs, scale_lds);
     } else {
-        seg_wide_item<GATE_UP, R, D, 1, SG>(gu, dn, s, blockIdx.x, xs, scale_lds);
+        seg_wide_item<GATE_UP, R, D, 1, SG, SL>(gu, dn, s, blockIdx.x, xs, scale_lds);
     }
 }
 
@@ -709,8 +718,16 @@ static void launch_seg_rds(const SegGateUpArgs& gu, const SegDownArgs& dn, int t
     const dim3 grid(tiles / R, capacity);
     if (k_split == 0) {
         const size_t scale_bytes = seg_wide_scale_lds_bytes(GATE_UP, R, GATE_UP ? gu.H : dn.I, SG);
-        a64_seg_wide_kernel<GATE_UP, R, D, SG>
-            <<<dim3(tiles / (4 * R), capacity), 256, scale_bytes, stream>>>(gu, dn);
+        const dim3 wide(tiles / (4 * R), capacity);
+        if constexpr (SG == 4) {
+            // four scales per group over a long K do not fit the workgroup's LDS: they come
+            // with the weight ring instead (two rows' worth of registers a group)
+            if (!seg_wide_fits(GATE_UP, R, GATE_UP ? gu.H : dn.I, SG)) {
+                a64_seg_wide_kernel<GATE_UP, R, (D > 2 ? 2 : D), SG, false><<<wide, 256, 0, stream>>>(gu, dn);
+                return;
+            }
+        }
+        a64_seg_wide_kernel<GATE_UP, R, D, SG, true><<<wide, 256, scale_bytes, stream>>>(gu, dn);
     } else if (k_split >= 4 && (GATE_UP ? gu.H : dn.I) >= 4 * 128) {
         a64_seg_kernel<GATE_UP, R, 4, D, SG><<<grid, 256, 0, stream>>>(gu, dn);
     } else if (k_split >= 2 && (GATE_UP ? gu.H : dn.I) >= 2 * 128) {
@@ -770,7 +787,8 @@ int launch_seg_gate_up(const SegGateUpArgs& a, int k_split, int row_tiles, int d
                  "rows 16-byte aligned (H=%d I=%d pitch=%ld)", a.H, a.I, a.x_stride);
     AEON_REQUIRE(a.scales_per_group == 1 || a.scales_per_group == 4, AEON_ERR_INVALID_ARGUMENT,
                  "gate/up segments: %d scales per 128 columns (1 or 4)", a.scales_per_group);
-    AEON_REQUIRE(k_split != 0 || seg_wide_fits(true, 1, a.H, a.scales_per_group), AEON_ERR_INVALID_ARGUMENT,
+    AEON_REQUIRE(k_split != 0 || a.scales_per_group == 4 || seg_wide_fits(true, 1, a.H, a.scales_per_group),
+                 AEON_ERR_INVALID_ARGUMENT,
                  "gate/up segments: the scales of %d columns do not fit the wide form's LDS", a.H);
     if (a.seg.capacity <= 0) return AEON_OK;
     launch_seg<true>(a, SegDownArgs{}, a.I / 16, a.seg.capacity, k_split, row_tiles, depth, stream);
@@ -783,7 +801,8 @@ int launch_seg_down(const SegDownArgs& a, int k_split, int row_tiles, int depth,
                  "down segments: need I%%128==0 and H%%16==0 (H=%d I=%d)", a.H, a.I);
     AEON_REQUIRE(a.scales_per_group == 1 || a.scales_per_group == 4, AEON_ERR_INVALID_ARGUMENT,
                  "down segments: %d scales per 128 columns (1 or 4)", a.scales_per_group);
-    AEON_REQUIRE(k_split != 0 || seg_wide_fits(false, 1, a.I, a.scales_per_group), AEON_ERR_INVALID_ARGUMENT,
+    AEON_REQUIRE(k_split != 0 || a.scales_per_group == 4 || seg_wide_fits(false, 1, a.I, a.scales_per_group),
+                 AEON_ERR_INVALID_ARGUMENT,
                  "down segments: the scales of %d columns do not fit the wide form's LDS", a.I);
     if (a.seg.capacity <= 0) return AEON_OK;
     launch_seg<false>(SegGateUpArgs{}, a, a.H / 16, a.seg.capacity, k_split, row_tiles, depth, stream);

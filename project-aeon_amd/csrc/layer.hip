@@ -187,14 +187,15 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
     // activations through LDS, no K split). Few: split K four ways so the chip still fills.
     // Measured at H 7168 / I 2048: the gate/up launch is faster K-split up to batch 2 (17 live
     // lists) and wide from batch 4 (33) on; the down launch is faster wide at every batch.
-    // The wide form also has to hold its tiles' scales over all of K in LDS; where four scales
-    // per 128 columns of a long K do not fit, the K-split form (scales straight from memory)
-    // serves every batch.
+    // The wide form holds its tiles' scales over all of K in LDS; where one scale per 128 columns
+    // of a long K does not fit, the K-split form (scales straight from memory) serves every
+    // batch. With four scales per 128 columns the wide form has a variant of its own for that
+    // case: the scales travel in the register ring with the weights.
     const int per_group = layer->scale_group == 32 ? 4 : 1;
     const int split_gate = live_bound * (layer->intermediate / 16) >= 3072 &&
-                                   seg_wide_fits(true, 1, layer->hidden, per_group) ? 0 : 4;
+                                   (per_group == 4 || seg_wide_fits(true, 1, layer->hidden, per_group)) ? 0 : 4;
     const int split_down = live_bound * (layer->hidden / 16) >= 4000 &&
-                                   seg_wide_fits(false, 1, layer->intermediate, per_group) ? 0 : 4;
+                                   (per_group == 4 || seg_wide_fits(false, 1, layer->intermediate, per_group)) ? 0 : 4;
     // Wide form: 64 gate/up rows or 128 down rows per workgroup and four (three) K groups of
     // weights in flight per wave measured best at batch 64 on both a concentrated and a spread
     // routing; more rows per workgroup save activation reads but leave fewer workgroups to
