@@ -720,9 +720,11 @@ static void launch_seg_rds(const SegGateUpArgs& gu, const SegDownArgs& dn, int t
         const size_t scale_bytes = seg_wide_scale_lds_bytes(GATE_UP, R, GATE_UP ? gu.H : dn.I, SG);
         const dim3 wide(tiles / (4 * R), capacity);
         if constexpr (SG == 4) {
-            // four scales per group over a long K do not fit the workgroup's LDS: they come
-            // with the weight ring instead (two rows' worth of registers a group)
-            if (!seg_wide_fits(GATE_UP, R, GATE_UP ? gu.H : dn.I, SG)) {
+            // Four scales per group: over a long K they do not fit the workgroup's LDS and come
+            // with the weight ring instead (two registers per tile and group in flight). The
+            // gate/up launch takes that form at every K: its LDS copy (32 KB at K 4096) would
+            // cost a workgroup per CU, and the ring form measured 1-3 % faster there.
+            if (GATE_UP || !seg_wide_fits(GATE_UP, R, GATE_UP ? gu.H : dn.I, SG)) {
                 a64_seg_wide_kernel<GATE_UP, R, (D > 2 ? 2 : D), SG, false><<<wide, 256, 0, stream>>>(gu, dn);
                 return;
             }
