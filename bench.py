@@ -354,6 +354,44 @@ def run_dropin(capi, moe, torch, np):
                                 "ms": round(ms, 4), "us_per_token": round(ms * 1e3 / T, 2),
                                 "weights_gbps": round(touched * expert_bytes / ms / 1e6, 1),
                                 "tflops": round(2.0 * T * K * 3 * H * I / ms / 1e9, 1)})
+
+    # The whole layer step as the checkpoint composes it (aeon_moe_layer_decode): fp16 gate
+    # [256 x 4096] with fp16 logits, sqrt(softplus) + bias, top-6 scaled by 1.5, the unquantised
+    # fp16 shared expert, the group-32 routed experts above, the slot-ordered reduce. Activations
+    # rotate so that the routed experts change from step to step.
+    gate = (torch.randn(NE, H, device="cuda", generator=gen) * 0.02).half()
+    bias = torch.randn(NE, device="cuda", generator=gen) * 0.05
+    dense = tuple((torch.randn(r, c, device="cuda", generator=gen) * 0.03).half()
+                  for r, c in ((I, H), (I, H), (H, I)))
+    layer = moe.MoeLayer(pool, NE, K, False, limit, None, bias, score_kind=0, routed_scaling_factor=1.5,
+                         router_weight_f16=gate, dense_shared=dense)
+    res["checkpoint_layer_step"] = []
+    dense_bytes = 3 * H * I * 2 + NE * H * 2
+    for T in (1, 8, 64):
+        xs = [(torch.rand(T, H, device="cuda", generator=gen) - 0.5).half() for _ in range(8)]
+        outb = torch.empty(T, H, dtype=torch.float16, device="cuda")
+        ids = torch.empty(T, K, dtype=torch.int32, device="cuda")
+        wts = torch.empty(T, K, dtype=torch.float32, device="cuda")
+
+        def step(i):
+            layer.decode(xs[i % 8], outb, ids, wts)
+
+        settle(step, torch)
+        a.record()
+        for i in range(200):
+            step(i)
+        b.record()
+        torch.cuda.synchronize()
+        ms = a.elapsed_time(b) / 200
+        touched = []
+        for r in range(8):
+            layer.decode(xs[r], outb, ids, wts)
+            torch.cuda.synchronize()
+            touched.append(int(torch.unique(ids).numel()))
+        moved = float(np.mean(touched)) * expert_bytes + dense_bytes
+        res["checkpoint_layer_step"].append({"tokens": T, "distinct_experts": round(float(np.mean(touched)), 1),
+                                             "ms": round(ms, 4), "us_per_token": round(ms * 1e3 / T, 2),
+                                             "bytes": int(moved), "gbps": round(moved / ms / 1e6, 1)})
     return res
 
 

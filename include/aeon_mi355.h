@@ -243,15 +243,17 @@ int aeon_router_logits_f16(const void* d_x, int x_stride, const void* d_gate_wei
 int aeon_dense_gemv_f16(const void* d_x, int x_stride, const void* d_weight, void* d_y,
                         int y_stride, int tokens, int in_dim, int out_dim, void* stream);
 /* run_layer_body_moe_shared_expert, layer/v4_layer_body_moe.hpp:216-256 (oracle: dense_ffn,
- * reference/dsv4_oracle.hpp:1708-1753), for `tokens` tokens in two launches: gate = half(W1 x),
- * up = half(W3 x) into d_gate / d_up ([tokens][intermediate] fp16, caller's scratch), then
- * out[t] = half(W2 . half(clamped_swiglu(gate, up))) -- the stage roundings of the reference's
- * four launches (three GEMVs and v4_swiglu_clamp_kernel). The reference's memset of the
- * accumulator is not needed: every element of the `hidden` columns of the output rows is written. */
+ * reference/dsv4_oracle.hpp:1708-1753), for `tokens` tokens in three launches: gate = half(W1 x)
+ * and up = half(W3 x) into d_gate / d_up, hidden = half(clamped_swiglu(gate, up)) into d_hidden
+ * (the reference's d_shared_gate / d_shared_up / d_shared_swiglu; each [tokens][intermediate]
+ * fp16, caller's scratch), then out[t] = half(W2 . hidden) -- the stage roundings of the
+ * reference's four launches (three GEMVs and v4_swiglu_clamp_kernel). The reference's memset of
+ * the accumulator is not needed: every element of the `hidden` columns of the output rows is
+ * written. intermediate % 128 == 0 and hidden % 128 == 0. */
 int aeon_dense_shared_expert_f16(const void* d_x, int x_stride, int tokens, const void* d_w1,
                                  const void* d_w3, const void* d_w2, void* d_gate, void* d_up,
-                                 void* d_out, int out_stride, int hidden, int intermediate,
-                                 float swiglu_limit, void* stream);
+                                 void* d_hidden, void* d_out, int out_stride, int hidden,
+                                 int intermediate, float swiglu_limit, void* stream);
 
 /* moe_router_kernel launch (src/architecture/deepseek_v4/kernels/moe_router.hpp:104-189; host
  * twin cpu_moe_router :29-100): score = f(logit); choice = score + bias (bias added after the

@@ -11,18 +11,15 @@
 // 128-column groups (wave w takes groups w, w+4, ...). Lane l supplies weight row l%16 / token
 // l%16 and columns 32s + 8(l/16)..+7 of step s, 16 bytes per load: a wave's four loads of a group
 // cover 256 contiguous bytes of each of its 16 rows. The lane ends up with rows 4(l/16)..+3 of
-// token l%16, an 8-byte store. Bound by the weight stream for a decode batch.
+// token l%16, an 8-byte store. Bound by the weight stream for a decode batch. The shared expert
+// is three launches: W1 and W3 (one grid, two matrices), the element-wise clamped SwiGLU, W2.
 #include "common.hpp"
 
 namespace aeon355 {
 
 struct DenseArgs {
-    const uint16_t* x;      // [tokens][x_stride] fp16; unused when the input is a SwiGLU of gate/up
+    const uint16_t* x;      // [tokens][x_stride] fp16
     long x_stride;
-    const uint16_t* gate;   // SwiGLU input: x[t][i] = half(clamped_swiglu(gate[t][i], up[t][i]))
-    const uint16_t* up;
-    long gu_stride;
-    float limit;
     const uint16_t* w[2];   // blockIdx.y picks the matrix: [out_dim][in_dim] row-major fp16
     uint16_t* y[2];         // [tokens][y_stride] fp16
     float* y32;             // optional (matrix 0): the fp16 result widened, [tokens][out_dim]
@@ -30,21 +27,28 @@ struct DenseArgs {
     int tokens, in_dim, out_dim;
 };
 
-__device__ __forceinline__ half8_t swiglu8(const u32x4_t& g, const u32x4_t& u, float limit) {
-    half8_t out;
+// hidden[t][i] = half(clamped_swiglu(gate[t][i], up[t][i])): the reference's
+// v4_swiglu_clamp_kernel between the shared expert's projections, eight elements a thread.
+__global__ __launch_bounds__(256) void dense_swiglu_kernel(const u32x4_t* __restrict__ gate,
+                                                           const u32x4_t* __restrict__ up,
+                                                           u32x4_t* __restrict__ hidden, int units,
+                                                           float limit) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= units) return;
+    const u32x4_t g = gate[i], u = up[i];
+    u32x4_t h;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const float g0 = half_bits_to_float(static_cast<uint16_t>(g[i] & 0xFFFFu));
-        const float g1 = half_bits_to_float(static_cast<uint16_t>(g[i] >> 16));
-        const float u0 = half_bits_to_float(static_cast<uint16_t>(u[i] & 0xFFFFu));
-        const float u1 = half_bits_to_float(static_cast<uint16_t>(u[i] >> 16));
-        out[2 * i] = static_cast<half_t>(clamped_swiglu(g0, u0, limit));
-        out[2 * i + 1] = static_cast<half_t>(clamped_swiglu(g1, u1, limit));
+    for (int q = 0; q < 4; ++q) {
+        const float lo = clamped_swiglu(half_bits_to_float(static_cast<uint16_t>(g[q] & 0xFFFFu)),
+                                        half_bits_to_float(static_cast<uint16_t>(u[q] & 0xFFFFu)), limit);
+        const float hi = clamped_swiglu(half_bits_to_float(static_cast<uint16_t>(g[q] >> 16)),
+                                        half_bits_to_float(static_cast<uint16_t>(u[q] >> 16)), limit);
+        h[q] = float_to_half_bits(lo) | (static_cast<uint32_t>(float_to_half_bits(hi)) << 16);
     }
-    return out;
+    hidden[i] = h;
 }
 
-template <int MT, bool SWIGLU>
+template <int MT>
 __global__ __launch_bounds__(256) void dense_f16_kernel(DenseArgs a) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -59,18 +63,11 @@ __global__ __launch_bounds__(256) void dense_f16_kernel(DenseArgs a) {
         as_global<uint16_t>(a.w[matrix]) + static_cast<size_t>(tile * 16 + n) * a.in_dim + chunk * 8;
     // a padded token column repeats the last live token: a valid row whose results are not stored
     const AEON_GLOBAL uint16_t* xrow[MT];
-    const AEON_GLOBAL uint16_t* urow[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         int token = token0 + mt * 16 + n;
         token = token < a.tokens ? token : a.tokens - 1;
-        if (SWIGLU) {
-            xrow[mt] = as_global<uint16_t>(a.gate) + token * a.gu_stride + chunk * 8;
-            urow[mt] = as_global<uint16_t>(a.up) + token * a.gu_stride + chunk * 8;
-        } else {
-            xrow[mt] = as_global<uint16_t>(a.x) + token * a.x_stride + chunk * 8;
-            urow[mt] = xrow[mt];
-        }
+        xrow[mt] = as_global<uint16_t>(a.x) + token * a.x_stride + chunk * 8;
     }
 
     float4_t acc[MT];
@@ -81,7 +78,6 @@ __global__ __launch_bounds__(256) void dense_f16_kernel(DenseArgs a) {
     constexpr int D = 2;
     u32x4_t wq[D][4];
     u32x4_t xq[D][MT][4];
-    u32x4_t uq[D][SWIGLU ? MT : 1][4];
     auto load_group = [&](int d, int g) {
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
@@ -89,9 +85,6 @@ __global__ __launch_bounds__(256) void dense_f16_kernel(DenseArgs a) {
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 xq[d][mt][st] = *reinterpret_cast<const AEON_GLOBAL u32x4_t*>(xrow[mt] + g * 128 + st * 32);
-                if (SWIGLU) {
-                    uq[d][mt][st] = *reinterpret_cast<const AEON_GLOBAL u32x4_t*>(urow[mt] + g * 128 + st * 32);
-                }
             }
         }
     };
@@ -103,11 +96,7 @@ __global__ __launch_bounds__(256) void dense_f16_kernel(DenseArgs a) {
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 union { u32x4_t u; half8_t h; } xf;
-                if (SWIGLU) {
-                    xf.h = swiglu8(xq[d][mt][st], uq[d][mt][st], a.limit);
-                } else {
-                    xf.u = xq[d][mt][st];
-                }
+                xf.u = xq[d][mt][st];
                 acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf.h, xf.h, acc[mt], 0, 0, 0);
             }
         }
@@ -169,16 +158,15 @@ __global__ __launch_bounds__(256) void dense_f16_kernel(DenseArgs a) {
     }
 }
 
-template <bool SWIGLU>
 static int launch_dense(const DenseArgs& a, int matrices, hipStream_t stream) {
     if (a.tokens <= 0) return AEON_OK;
     const int tiles = a.out_dim / 16;
     if (a.tokens <= 16) {
-        dense_f16_kernel<1, SWIGLU><<<dim3(tiles, matrices, 1), 256, 0, stream>>>(a);
+        dense_f16_kernel<1><<<dim3(tiles, matrices, 1), 256, 0, stream>>>(a);
     } else if (a.tokens <= 32) {
-        dense_f16_kernel<2, SWIGLU><<<dim3(tiles, matrices, 1), 256, 0, stream>>>(a);
+        dense_f16_kernel<2><<<dim3(tiles, matrices, 1), 256, 0, stream>>>(a);
     } else {
-        dense_f16_kernel<4, SWIGLU><<<dim3(tiles, matrices, (a.tokens + 63) / 64), 256, 0, stream>>>(a);
+        dense_f16_kernel<4><<<dim3(tiles, matrices, (a.tokens + 63) / 64), 256, 0, stream>>>(a);
     }
     AEON_LAUNCH_CHECK();
     return AEON_OK;
@@ -204,13 +192,14 @@ int launch_dense_gemv(const void* d_x, long x_stride, const void* d_w, void* d_y
     a.tokens = tokens;
     a.in_dim = in_dim;
     a.out_dim = out_dim;
-    return launch_dense<false>(a, 1, stream);
+    return launch_dense(a, 1, stream);
 }
 
 int launch_dense_shared_expert(const void* d_x, long x_stride, int tokens, const void* d_w1,
                                const void* d_w3, const void* d_w2, void* d_gate, void* d_up,
-                               void* d_out, long out_stride, int hidden, int intermediate, float limit,
-                               hipStream_t stream) {
+                               void* d_hidden, void* d_out, long out_stride, int hidden,
+                               int intermediate, float limit, hipStream_t stream) {
+    if (tokens <= 0) return AEON_OK;
     DenseArgs gu{};
     gu.x = static_cast<const uint16_t*>(d_x);
     gu.x_stride = x_stride;
@@ -222,19 +211,24 @@ int launch_dense_shared_expert(const void* d_x, long x_stride, int tokens, const
     gu.tokens = tokens;
     gu.in_dim = hidden;
     gu.out_dim = intermediate;
-    if (int rc = launch_dense<false>(gu, 2, stream)) return rc;
+    if (int rc = launch_dense(gu, 2, stream)) return rc;
+    // the activation is applied once, between the launches: inside the W2 launch every one of
+    // its row-tile workgroups would redo it for all of the tokens' columns
+    const int units = tokens * (intermediate / 8);
+    dense_swiglu_kernel<<<(units + 255) / 256, 256, 0, stream>>>(
+        static_cast<const u32x4_t*>(d_gate), static_cast<const u32x4_t*>(d_up),
+        static_cast<u32x4_t*>(d_hidden), units, limit);
+    AEON_LAUNCH_CHECK();
     DenseArgs dn{};
-    dn.gate = static_cast<const uint16_t*>(d_gate);
-    dn.up = static_cast<const uint16_t*>(d_up);
-    dn.gu_stride = intermediate;
-    dn.limit = limit;
+    dn.x = static_cast<const uint16_t*>(d_hidden);
+    dn.x_stride = intermediate;
     dn.w[0] = static_cast<const uint16_t*>(d_w2);
     dn.y[0] = static_cast<uint16_t*>(d_out);
     dn.y_stride = out_stride;
     dn.tokens = tokens;
     dn.in_dim = intermediate;
     dn.out_dim = hidden;
-    return launch_dense<true>(dn, 1, stream);
+    return launch_dense(dn, 1, stream);
 }
 
 }  // namespace aeon355
@@ -255,19 +249,20 @@ extern "C" int aeon_dense_gemv_f16(const void* d_x, int x_stride, const void* d_
 
 extern "C" int aeon_dense_shared_expert_f16(const void* d_x, int x_stride, int tokens,
                                             const void* d_w1, const void* d_w3, const void* d_w2,
-                                            void* d_gate, void* d_up, void* d_out, int out_stride,
-                                            int hidden, int intermediate, float swiglu_limit,
-                                            void* stream) {
+                                            void* d_gate, void* d_up, void* d_hidden, void* d_out,
+                                            int out_stride, int hidden, int intermediate,
+                                            float swiglu_limit, void* stream) {
     const char* who = "aeon_dense_shared_expert_f16";
-    AEON_REQUIRE(d_x && d_w1 && d_w3 && d_w2 && d_gate && d_up && d_out, AEON_ERR_INVALID_ARGUMENT,
+    AEON_REQUIRE(d_x && d_w1 && d_w3 && d_w2 && d_gate && d_up && d_hidden && d_out, AEON_ERR_INVALID_ARGUMENT,
                  "%s: null buffer", who);
     if (int rc = check_dense_shape(tokens, hidden, intermediate, who)) return rc;
     if (int rc = check_dense_shape(tokens, intermediate, hidden, who)) return rc;
     AEON_REQUIRE(x_stride >= hidden && x_stride % 8 == 0 && out_stride >= hidden && out_stride % 4 == 0,
                  AEON_ERR_INVALID_ARGUMENT, "%s: bad row pitch (x_stride=%d out_stride=%d)", who, x_stride,
                  out_stride);
-    return launch_dense_shared_expert(d_x, x_stride, tokens, d_w1, d_w3, d_w2, d_gate, d_up, d_out,
-                                      out_stride, hidden, intermediate, swiglu_limit, as_stream(stream));
+    return launch_dense_shared_expert(d_x, x_stride, tokens, d_w1, d_w3, d_w2, d_gate, d_up, d_hidden,
+                                      d_out, out_stride, hidden, intermediate, swiglu_limit,
+                                      as_stream(stream));
 }
 
 extern "C" int aeon_router_logits_f16(const void* d_x, int x_stride, const void* d_gate_weight,

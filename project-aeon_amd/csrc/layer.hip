@@ -19,8 +19,8 @@ int launch_dense_gemv(const void* d_x, long x_stride, const void* d_w, void* d_y
                       float* d_y32, int tokens, int in_dim, int out_dim, hipStream_t stream);
 int launch_dense_shared_expert(const void* d_x, long x_stride, int tokens, const void* d_w1,
                                const void* d_w3, const void* d_w2, void* d_gate, void* d_up,
-                               void* d_out, long out_stride, int hidden, int intermediate, float limit,
-                               hipStream_t stream);
+                               void* d_hidden, void* d_out, long out_stride, int hidden,
+                               int intermediate, float limit, hipStream_t stream);
 
 // Up to this many tokens a step always runs on the weight-streaming (decode) kernels. Above it
 // the grouped GEMM takes over once the experts hold enough positions each for its windows to
@@ -52,6 +52,7 @@ struct LayerWorkspace {
     float* contrib;
     uint16_t* dense_gate;   // [tokens][intermediate] fp16 each, for a dense shared expert
     uint16_t* dense_up;
+    uint16_t* dense_hidden;
     int positions;
     int seg_capacity;
     size_t bytes;
@@ -89,6 +90,7 @@ static LayerWorkspace carve(const aeon_moe_layer& L, int tokens, void* base) {
     const size_t dense_bytes = dense_shared ? sizeof(uint16_t) * static_cast<size_t>(tokens) * L.intermediate : 0;
     w.dense_gate = reinterpret_cast<uint16_t*>(take(dense_bytes));
     w.dense_up = reinterpret_cast<uint16_t*>(take(dense_bytes));
+    w.dense_hidden = reinterpret_cast<uint16_t*>(take(dense_bytes));
     w.bytes = at;
     return w;
 }
@@ -235,7 +237,7 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
                      "%s: the dense shared expert stores 8 bytes at a time (out_stride=%d)", who, out_stride);
         if (int rc = launch_dense_shared_expert(d_x, x_stride, tokens, layer->d_shared_w1_f16,
                                                 layer->d_shared_w3_f16, layer->d_shared_w2_f16,
-                                                w.dense_gate, w.dense_up, d_out, out_stride,
+                                                w.dense_gate, w.dense_up, w.dense_hidden, d_out, out_stride,
                                                 layer->hidden, layer->intermediate,
                                                 layer->swiglu_limit, s)) {
             return rc;

@@ -69,16 +69,23 @@ def test_dense_shared_expert_against_the_oracle(orc, tokens, hidden, inter, limi
     dev = [h.dev_half(a) for a in (x, w1, w3, w2)]
     gate = torch.zeros(tokens, inter, dtype=torch.float16, device="cuda")
     up = torch.zeros_like(gate)
+    act = torch.zeros_like(gate)
     out = torch.full((tokens, hidden), 5.0, dtype=torch.float16, device="cuda")   # stale accumulator
     capi.call("aeon_dense_shared_expert_f16", capi.vp(dev[0]), hidden, tokens, capi.vp(dev[1]),
-              capi.vp(dev[2]), capi.vp(dev[3]), capi.vp(gate), capi.vp(up), capi.vp(out), hidden, hidden,
-              inter, C.c_float(limit), h.stream_ptr())
+              capi.vp(dev[2]), capi.vp(dev[3]), capi.vp(gate), capi.vp(up), capi.vp(act), capi.vp(out),
+              hidden, hidden, inter, C.c_float(limit), h.stream_ptr())
     got = out.cpu().numpy().astype(np.float64)
     w64 = [a.astype(np.float64) for a in (w1, w3, w2)]
     # stage by stage: gate and up are single GEMVs
     ex, near = _one_rounding(gate.cpu().numpy(), x.astype(np.float64) @ w64[0].T)
     assert np.all(ex | near)
     ex, near = _one_rounding(up.cpu().numpy(), x.astype(np.float64) @ w64[1].T)
+    assert np.all(ex | near)
+    # the activation stage on the device's own gate and up: one rounding of the fp64 value
+    g16, u16 = gate.cpu().numpy().astype(np.float64).ravel(), up.cpu().numpy().astype(np.float64).ravel()
+    pick = rng.choice(g16.size, size=min(4000, g16.size), replace=False)
+    want = np.array([orc.clamped_swiglu(g16[i], u16[i], limit) for i in pick])
+    ex, near = _one_rounding(act.cpu().numpy().ravel()[pick], want)
     assert np.all(ex | near)
     # the composed FFN: the device's view (stages stored as fp16) and the oracle's own (no
     # rounding between stages, dense_ffn as the reference states it)
