@@ -59,17 +59,28 @@ __global__ __launch_bounds__(256) void dense_f16_kernel(DenseArgs a) {
     const int token0 = blockIdx.z * 16 * MT;
     const int groups = a.in_dim / 128;
 
+    // Loads: lane l fetches 16 bytes of row l/4 at 16-byte piece l%4, so four neighbouring lanes
+    // read 64 contiguous bytes (the matrix instruction's own lane order, row l%16 / piece l/16,
+    // would make every lane a separate cache access: 64 per wave load instead of 16). The
+    // fragments change lanes on their way into the MFMA,
+    const int lrow = lane >> 2;
+    const int lpiece = lane & 3;
+    // through a wave-private LDS tile of 16 rows x 64 bytes (pitch 80 bytes: both the write in
+    // load order and the read in MFMA order touch every bank evenly); LDS serves a wave's
+    // accesses in order, so the wave needs no barrier between its write and its read
+    __shared__ u32x4_t stage[4][2][(1 + MT) * 80];
+    const int put = lrow * 5 + lpiece;
+    const int take = n * 5 + chunk;
     const AEON_GLOBAL uint16_t* wrow =
-        as_global<uint16_t>(a.w[matrix]) + static_cast<size_t>(tile * 16 + n) * a.in_dim + chunk * 8;
+        as_global<uint16_t>(a.w[matrix]) + static_cast<size_t>(tile * 16 + lrow) * a.in_dim + lpiece * 8;
     // a padded token column repeats the last live token: a valid row whose results are not stored
     const AEON_GLOBAL uint16_t* xrow[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-        int token = token0 + mt * 16 + n;
+        int token = token0 + mt * 16 + lrow;
         token = token < a.tokens ? token : a.tokens - 1;
-        xrow[mt] = as_global<uint16_t>(a.x) + token * a.x_stride + chunk * 8;
+        xrow[mt] = as_global<uint16_t>(a.x) + token * a.x_stride + lpiece * 8;
     }
-
     float4_t acc[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
@@ -91,13 +102,19 @@ __global__ __launch_bounds__(256) void dense_f16_kernel(DenseArgs a) {
     auto compute = [&](int d) {
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
-            union { u32x4_t u; half8_t h; } wf;
-            wf.u = wq[d][st];
+            u32x4_t* tile_slot = stage[wave][st & 1];
+            tile_slot[put] = wq[d][st];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) tile_slot[(1 + mt) * 80 + put] = xq[d][mt][st];
+            asm volatile("" ::: "memory");
+            union { u32x4_t u; half8_t h; } wf, xf[MT];
+            wf.u = tile_slot[take];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) xf[mt].u = tile_slot[(1 + mt) * 80 + take];
+            asm volatile("" ::: "memory");
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-                union { u32x4_t u; half8_t h; } xf;
-                xf.u = xq[d][mt][st];
-                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf.h, xf.h, acc[mt], 0, 0, 0);
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf.h, xf[mt].h, acc[mt], 0, 0, 0);
             }
         }
     };
