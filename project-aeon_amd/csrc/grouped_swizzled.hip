@@ -66,21 +66,31 @@ __device__ __forceinline__ void grouped_swizzled_window(const GroupedSwzArgs& a,
     const uint16_t* sb = GATE_UP ? static_cast<const uint16_t*>(a.w13.s3[expert]) : nullptr;
 
     // a padded token column repeats the window's last live position; its results are not stored
+    // A pass's image in LDS is [token tile][step j][lane (token n, 32-group chunk)], 16 bytes
+    // each = columns 32 chunk + 8 j..+7 of the pass. Wave w fetches 32-group w of it in row
+    // order: lane l takes 16-byte piece l%4 of token l/4, four neighbouring lanes 64 contiguous
+    // bytes (16 cache accesses per load; one lane per (token, piece) pair in the image's own lane
+    // order would be 64), and writes it to (step l%4, token l/4, chunk w).
+    const int load_token = lane >> 2;
+    const int load_step = lane & 3;
     const uint16_t* xrow[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-        const int m = m0 + mt * 16 + n < count ? m0 + mt * 16 + n : count - 1;
+        const int m = m0 + mt * 16 + load_token < count ? m0 + mt * 16 + load_token : count - 1;
         if (GATE_UP) {
             xrow[mt] = a.activation + static_cast<size_t>(a.token_indices[first + m]) * a.activation_stride;
         } else {
             xrow[mt] = a.activation + (static_cast<size_t>(expert) * a.hidden_tokens + m) * a.K;
         }
-        xrow[mt] += chunk * 32 + wave * 8;   // this wave's step of this lane's slot
+        xrow[mt] += wave * 32 + load_step * 8;
     }
     auto x_fragment = [&](int mt, int G) {
         return *reinterpret_cast<const half8_t*>(xrow[mt] + G * 128);
     };
     auto lds = [&](int buffer, int mt, int j) { return xs + ((buffer * kSwzWindowTiles + mt) * 4 + j) * 64 + lane; };
+    auto lds_put = [&](int buffer, int mt) {
+        return xs + ((buffer * kSwzWindowTiles + mt) * 4 + load_step) * 64 + wave * 16 + load_token;
+    };
 
     const size_t slot_base = (static_cast<size_t>(row / RPW) * iterations) * 32 + (row % RPW) * LPR;
     auto slot_of = [&](int G) {
@@ -139,7 +149,7 @@ __device__ __forceinline__ void grouped_swizzled_window(const GroupedSwzArgs& a,
         for (int mt = 0; mt < MT; ++mt) xr[slot][mt] = x_fragment(mt, G < passes ? G : passes - 1);
     };
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) *lds(0, mt, wave) = x_fragment(mt, 0);
+    for (int mt = 0; mt < MT; ++mt) *lds_put(0, mt) = x_fragment(mt, 0);
     // the requests before the loop go out in the loop's order (the fragments a pass fetches,
     // then the weights it fetches): the compiler's wait counts are static
 #pragma unroll
@@ -179,7 +189,7 @@ __device__ __forceinline__ void grouped_swizzled_window(const GroupedSwzArgs& a,
         }
         const int next_slot = kAhead == 1 ? 0 : (d + 1) % kAhead;
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) *lds((G + 1) & 1, mt, wave) = xr[next_slot][mt];
+        for (int mt = 0; mt < MT; ++mt) *lds_put((G + 1) & 1, mt) = xr[next_slot][mt];
         fetch_x(next_slot, G + 1 + kAhead);   // past the end: the last pass again, unused
         fetch_weights(d, G + kDepth);
         __syncthreads();
