@@ -8,10 +8,11 @@
 // then a fixed-order sum over the four waves that split K), the roundings do not.
 //
 // One workgroup = one 16-row tile of one matrix x up to 16*MT tokens; its four waves split K in
-// 128-column groups (wave w takes groups w, w+4, ...). Lane l supplies weight row l%16 / token
-// l%16 and columns 32s + 8(l/16)..+7 of step s, 16 bytes per load: a wave's four loads of a group
-// cover 256 contiguous bytes of each of its 16 rows. The lane ends up with rows 4(l/16)..+3 of
-// token l%16, an 8-byte store. Bound by the weight stream for a decode batch. The shared expert
+// 128-column groups (wave w takes groups w, w+4, ...). To the matrix instruction lane l supplies
+// weight row l%16 / token l%16 and columns 32s + 8(l/16)..+7 of step s; the loads are issued in
+// row order instead (lane l: row l/4, 16-byte piece l%4 of the step's 64 bytes) and the
+// fragments change lanes through LDS. The lane ends up with rows 4(l/16)..+3 of token l%16, an
+// 8-byte store. Bound by the weight stream for a decode batch. The shared expert
 // is three launches: W1 and W3 (one grid, two matrices), the element-wise clamped SwiGLU, W2.
 #include "common.hpp"
 

@@ -41,8 +41,8 @@ constexpr int kSwzWindowTiles = 4;  // token tiles of 16 positions one workgroup
 // cover the lane's slot, the four chunks cover the 128 columns.
 //
 // The four waves of a workgroup hold different weight rows and the same activations, so each
-// wave fetches one step's activation fragments (j = its index) a group ahead and all four read
-// them from LDS: one barrier per 128 columns, two LDS buffers (the one written in pass G was
+// wave fetches a quarter of the pass's activation fragments (32-group w for wave w, in row
+// order) a group ahead and all four read them from LDS: one barrier per 128 columns, two LDS buffers (the one written in pass G was
 // last read in pass G-1, before that pass's barrier). Weights and scales wait in a register
 // ring three passes deep, six for windows of one or two token tiles.
 template <int RPW, int LPR, bool GATE_UP, int MT>
