@@ -57,6 +57,32 @@ def test_dense_gemv_against_fp64(orc, tokens, in_dim, out_dim):
     assert torch.equal(again[:tokens], y[:tokens])          # fixed summation order
 
 
+@pytest.mark.parametrize("tokens,in_dim,out_dim,x_pitch,y_pitch", [(3, 384, 48, 392, 52), (20, 640, 32, 768, 40),
+                                                                    (64, 1152, 80, 1160, 96), (130, 384, 16, 512, 20)])
+def test_dense_gemv_with_row_pitches_and_uneven_k_shares(orc, tokens, in_dim, out_dim, x_pitch, y_pitch):
+    """Rows wider than the matrices (x_stride > in_dim, y_stride > out_dim) and a K whose 128-column
+    groups do not divide among the four waves: the columns between rows stay untouched and the
+    result is the compact call's, bit for bit."""
+    torch, h, capi, moe, synth = _setup()
+    rng = np.random.default_rng(tokens * 11 + in_dim)
+    w = rng.normal(0, 0.05, (out_dim, in_dim)).astype(np.float16)
+    x = rng.normal(0, 1, (tokens, in_dim)).astype(np.float16)
+    wide = np.full((tokens, x_pitch), np.float16(777.0))
+    wide[:, :in_dim] = x
+    d_w, d_x, d_wide = h.dev_half(w), h.dev_half(x), h.dev_half(wide)
+    compact = torch.zeros((tokens, out_dim), dtype=torch.float16, device="cuda")
+    capi.call("aeon_dense_gemv_f16", capi.vp(d_x), in_dim, capi.vp(d_w), capi.vp(compact), out_dim, tokens,
+              in_dim, out_dim, h.stream_ptr())
+    pitched = torch.full((tokens, y_pitch), 9.0, dtype=torch.float16, device="cuda")
+    capi.call("aeon_dense_gemv_f16", capi.vp(d_wide), x_pitch, capi.vp(d_w), capi.vp(pitched), y_pitch, tokens,
+              in_dim, out_dim, h.stream_ptr())
+    assert torch.equal(pitched[:, :out_dim], compact)
+    assert torch.all(pitched[:, out_dim:] == 9.0)
+    want = x.astype(np.float64) @ w.astype(np.float64).T
+    exact, near = _one_rounding(compact.cpu().numpy(), want)
+    assert np.all(exact | near)
+
+
 @pytest.mark.parametrize("tokens,hidden,inter,limit", [(1, 4096, 2048, 10.0), (7, 4096, 2048, 10.0),
                                                        (40, 1024, 512, 0.5), (70, 512, 256, 10.0)])
 def test_dense_shared_expert_against_the_oracle(orc, tokens, hidden, inter, limit):
