@@ -23,22 +23,34 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
 }
 
 // Exclusive scan of one value per thread across a 1024-thread workgroup.
-__device__ __forceinline__ int block_exclusive_scan(int v, int* wave_totals, int* total) {
+// Three scans in one: a list's position count (bits 0..23), its full segments (24..43) and its
+// short one (44..63) ride in one 64-bit word, so the segment list costs no barriers of its own.
+__device__ __forceinline__ unsigned long long block_exclusive_scan3(unsigned long long v,
+                                                                    unsigned long long* wave_totals,
+                                                                    unsigned long long* total) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int inclusive = wave_inclusive_scan(v, lane);
+    unsigned long long inclusive = v;
+#pragma unroll
+    for (int offset = 1; offset < 64; offset <<= 1) {
+        const unsigned long long other = __shfl_up(inclusive, offset, 64);
+        if (lane >= offset) inclusive += other;
+    }
     if (lane == 63) wave_totals[wave] = inclusive;
     __syncthreads();
     if (wave == 0) {
-        const int t = lane < 16 ? wave_totals[lane] : 0;
-        const int scanned = wave_inclusive_scan(t, lane);
+        const unsigned long long t = lane < 16 ? wave_totals[lane] : 0ull;
+        unsigned long long scanned = t;
+#pragma unroll
+        for (int offset = 1; offset < 16; offset <<= 1) {
+            const unsigned long long other = __shfl_up(scanned, offset, 64);
+            if (lane >= offset) scanned += other;
+        }
         if (lane < 16) wave_totals[lane] = scanned - t;
         if (lane == 15) *total = scanned;
     }
     __syncthreads();
-    const int result = inclusive - v + wave_totals[wave];
-    __syncthreads();
-    return result;
+    return inclusive - v + wave_totals[wave];
 }
 
 // A batch of at most this many draws is scattered by the workgroup that counts it (one launch
@@ -50,21 +62,26 @@ constexpr int kWaveCountWords = (kFusedScatterDraws / 64) * (kMaxPermutationExpe
 // Stable rank of each of a 1024-thread workgroup's draws among the workgroup's draws of the same
 // expert: thread i holds draw i of the chunk (`mine` = its expert, -1 for none), wave w the draws
 // 64w..64w+63. The earlier waves' share comes from per-wave counts in LDS (`wave_count`, zeroed
-// here), the share of the lower lanes from a walk over the wave's own 64 draws. Ends with the
-// workgroup synchronised.
+// here), the share of the lower lanes from the set of the wave's lanes with the same expert. Ends
+// with the workgroup synchronised.
 __device__ __forceinline__ int rank_in_chunk(int mine, int lists, uint32_t* wave_count_words) {
     unsigned short* wave_count = reinterpret_cast<unsigned short*>(wave_count_words);
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     for (int i = threadIdx.x; i < (16 * lists + 1) / 2; i += blockDim.x) wave_count_words[i] = 0;
     __syncthreads();
-    int rank = 0, later = 0;
-#pragma unroll 8
-    for (int l = 0; l < 64; ++l) {
-        const bool same = __builtin_amdgcn_readlane(mine, l) == mine;
-        rank += (l < lane && same) ? 1 : 0;
-        later += (l > lane && same) ? 1 : 0;
+    // the lanes of the wave that hold the same list: one ballot per bit of the id (a list index
+    // is at most kMaxPermutationExperts, 11 bits) and one for "no draw"
+    static_assert(kMaxPermutationExperts < (1 << 11), "the ballots cover 11 bits of a list index");
+    unsigned long long same = ~0ull;
+#pragma unroll
+    for (int b = 0; b <= 11; ++b) {
+        const bool set = b < 11 ? ((mine >> b) & 1) != 0 : mine < 0;
+        const unsigned long long ballot = __ballot(set);
+        same &= set ? ballot : ~ballot;
     }
+    int rank = __popcll(same & ((1ull << lane) - 1ull));
+    const int later = __popcll(same & ~((2ull << lane) - 1ull));
     // the last lane of an expert in the wave knows the wave's count for it
     if (mine >= 0 && later == 0) wave_count[wave * lists + mine] = static_cast<unsigned short>(rank + 1);
     __syncthreads();
@@ -77,8 +94,8 @@ __device__ __forceinline__ int rank_in_chunk(int mine, int lists, uint32_t* wave
 template <bool SCATTER>
 __global__ __launch_bounds__(1024) void permutation_offsets_kernel(PermutationArgs a) {
     __shared__ int histogram[kMaxPermutationExperts + 1];
-    __shared__ int wave_totals[16];
-    __shared__ int total;
+    __shared__ unsigned long long wave_totals[16];
+    __shared__ unsigned long long total;
     __shared__ int draw_expert[SCATTER ? kFusedScatterDraws : 1];
     const int lists = a.experts + (a.shared_tokens > 0 ? 1 : 0);
     for (int e = threadIdx.x; e <= kMaxPermutationExperts; e += blockDim.x) histogram[e] = 0;
@@ -94,23 +111,28 @@ __global__ __launch_bounds__(1024) void permutation_offsets_kernel(PermutationAr
 
     const int e = threadIdx.x;
     const int count = e < lists ? histogram[e] : 0;
-    const int offset = block_exclusive_scan(count, wave_totals, &total);
+    // Segments that are more than half full come first in the list, the short ones after
+    // them: the launches walk the list in order, so the costliest workgroups are dispatched
+    // first and the launch's tail is made of cheap ones.
+    const bool with_segments = a.seg_expert != nullptr;
+    const int segments = with_segments ? (count + a.seg_tokens - 1) / a.seg_tokens : 0;
+    const int last_count = count - (segments - 1) * a.seg_tokens;
+    const int light = segments > 0 && 2 * last_count <= a.seg_tokens ? 1 : 0;
+    const int heavy = segments - light;
+    const unsigned long long packed = static_cast<unsigned long long>(count) |
+                                      (static_cast<unsigned long long>(heavy) << 24) |
+                                      (static_cast<unsigned long long>(light) << 44);
+    const unsigned long long before = block_exclusive_scan3(packed, wave_totals, &total);
+    const unsigned long long sums = total;
+    const int offset = static_cast<int>(before & 0xFFFFFFull);
     if (e < lists) a.offsets[e] = offset;
-    if (e == 0) a.offsets[lists] = total;
+    if (e == 0) a.offsets[lists] = static_cast<int>(sums & 0xFFFFFFull);
 
-    if (a.seg_expert != nullptr) {
-        // Segments that are more than half full come first in the list, the short ones after
-        // them: the launches walk the list in order, so the costliest workgroups are dispatched
-        // first and the launch's tail is made of cheap ones.
-        const int segments = (count + a.seg_tokens - 1) / a.seg_tokens;
-        const int last_count = count - (segments - 1) * a.seg_tokens;
-        const int light = segments > 0 && 2 * last_count <= a.seg_tokens ? 1 : 0;
-        const int heavy = segments - light;
-        int heavy_total = 0;
-        const int heavy_base = block_exclusive_scan(heavy, wave_totals, &total);
-        heavy_total = total;
-        const int light_base = block_exclusive_scan(light, wave_totals, &total);
-        const int all = heavy_total + total;
+    if (with_segments) {
+        const int heavy_base = static_cast<int>((before >> 24) & 0xFFFFFull);
+        const int light_base = static_cast<int>(before >> 44);
+        const int heavy_total = static_cast<int>((sums >> 24) & 0xFFFFFull);
+        const int all = heavy_total + static_cast<int>(sums >> 44);
         for (int s = 0; s < segments; ++s) {
             const int at = s < heavy ? heavy_base + s : heavy_total + light_base;
             if (at < a.seg_capacity) {
