@@ -209,10 +209,20 @@ __global__ __launch_bounds__(256 * kParts) void router_topk_kernel(
             if (e < experts) {
                 int rank = 0;
                 const double mine = choice_lds[e];
-                for (int f = first; f < last; ++f) {
+                // A candidate f beats e when its score is higher, or equal with f < e. The wave's
+                // experts are 64 consecutive indices: for the candidates below all of them the
+                // test is one >=, for those above all of them one >, and only the 64 candidates
+                // in between need the index (the three loops' bounds are the same for the wave).
+                const int wave_lo = e - static_cast<int>(threadIdx.x & 63);
+                const int begin = min(first, last);   // a part past the last expert has no range
+                const int below_end = min(last, max(begin, wave_lo));
+                const int above_begin = max(below_end, min(last, wave_lo + 64));
+                for (int f = begin; f < below_end; ++f) rank += choice_lds[f] >= mine ? 1 : 0;
+                for (int f = below_end; f < above_begin; ++f) {
                     const double other = choice_lds[f];
                     rank += (other > mine || (other == mine && f < e)) ? 1 : 0;
                 }
+                for (int f = above_begin; f < last; ++f) rank += choice_lds[f] > mine ? 1 : 0;
                 if (kParts > 1) atomicAdd(&rank_lds[e], rank);
                 else rank_lds[e] = rank;
             }
