@@ -208,3 +208,48 @@ def test_layer_step_with_the_checkpoint_pieces(orc, T):
         assert np.abs(shared).max() > 0.05 * np.abs(want).max()
     out2, _, _ = layer.decode(d_x)
     assert torch.equal(out2, out)
+
+
+@pytest.mark.parametrize("T", [1, 6, 40, 150])
+def test_checkpoint_step_equals_its_routed_half_and_replays_from_a_graph(orc, T):
+    """With the fp16 gate and the dense shared expert the full step and the routed entry point
+    (given the step's own ids and weights) run the same expert kernels: same bits. The step is
+    also captured into a graph and replayed with new activations and eager steps in between;
+    every replay has to give the eager bits."""
+    torch, h, capi, moe, synth = _setup()
+    H, I, E, k, limit = 1024, 512, 32, 4, 10.0
+    pool = moe.ExpertPool(E, H, I, scale_group=32)
+    assert pool.fill_synthetic(seed=52, first_expert_id=0) == 0
+    rng = np.random.default_rng(52)
+    gate_w = rng.normal(0, 0.03, (E, H)).astype(np.float16)
+    bias = rng.normal(0, 0.05, E).astype(np.float32)
+    d_sw = [h.dev_half(rng.normal(0, 0.06, s).astype(np.float16)) for s in ((I, H), (I, H), (H, I))]
+    layer = moe.MoeLayer(pool, E, k, False, limit, None, h.to_dev(bias), score_kind=0, routed_scaling_factor=1.5,
+                         router_weight_f16=h.dev_half(gate_w), dense_shared=tuple(d_sw))
+    xs = [h.dev_half(synth.activations(52, T, H, unit=r)) for r in range(3)]
+    eager = []
+    for x in xs:
+        out, ids, w = layer.decode(x)
+        alone = layer.routed(x, ids, w)
+        torch.cuda.synchronize()
+        assert torch.equal(out, alone)
+        assert float(out.float().abs().max()) > 0.0
+        eager.append((out.clone(), ids.clone(), w.clone()))
+    x_in = xs[0].clone()
+    out = torch.full((T, H), 5.0, dtype=torch.float16, device="cuda")
+    ids = torch.empty(T, k, dtype=torch.int32, device="cuda")
+    w = torch.empty(T, k, dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        layer.decode(x_in, out, ids, w)
+    for r in (2, 0, 1, 2):
+        x_in.copy_(xs[r])
+        out.fill_(5.0)
+        between = layer.decode(xs[(r + 1) % 3])      # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager[r][0]), (T, r)
+        assert torch.equal(ids, eager[r][1]) and torch.equal(w, eager[r][2]), (T, r)
+        assert torch.equal(between[0], eager[(r + 1) % 3][0])
