@@ -94,6 +94,32 @@ def calibrate_read(capi, torch):
     return out
 
 
+def calibrate_lds(capi, torch):
+    """Cost of a 16-byte-per-lane LDS read of a 1 KiB fragment by the order the lanes address it
+    in (nanoseconds per wave-wide read and CU, every read waited for): their own order, the matrix
+    instruction's lanes on a position-major fragment, and the same with the pieces rotated."""
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    wgs = cus * 4
+    sink = torch.empty(wgs * 256, dtype=torch.int32, device="cuda")
+    out = {"cus": cus}
+    names = ("linear", "position_major", "position_major_rotated_by_half_n", "position_major_rotated_by_quarter_n")
+    for pattern, name in enumerate(names):
+        reads = C.c_double(0.0)
+
+        def launch(i=0):
+            capi.call("aeon_calibrate_lds_read", pattern, 2000, wgs, capi.vp(sink), C.c_size_t(sink.numel()),
+                      C.byref(reads), None)
+        settle(launch, torch, seconds=0.2)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(5):
+            launch()
+        b.record()
+        torch.cuda.synchronize()
+        out["ns_per_wave_read_per_cu_" + name] = round(a.elapsed_time(b) * 1e6 / (reads.value * 5 / cus), 2)
+    return out
+
+
 def calibrate_mfma(capi, torch):
     """Sustained fp16 matrix-pipe rates of this GPU, for reading the prefill figure: the
     library's register-resident MFMA loop (two waves per SIMD) with constant and with random
@@ -676,6 +702,8 @@ def main():
                          "the FETCH_SIZE / WRITE_SIZE counters are scaled by")
     ap.add_argument("--calibrate-read", action="store_true",
                     help="time a read-only stream over 1.5 GiB and exit")
+    ap.add_argument("--calibrate-lds", action="store_true",
+                    help="time 16-byte LDS reads of a fragment in four lane orders and print the result")
     ap.add_argument("--calibrate-mfma", action="store_true",
                     help="only measure the sustained fp16 MFMA rate (register-resident loop with "
                          "constant and with random operands) and a library fp16 GEMM, for context")
@@ -735,6 +763,9 @@ def main():
         return
     if args.calibrate_read:
         print(json.dumps(calibrate_read(capi, torch)))
+        return
+    if args.calibrate_lds:
+        print(json.dumps(calibrate_lds(capi, torch)))
         return
     if args.dropin:
         print(json.dumps({"dropin": run_dropin(capi, moe, torch, np)}))

@@ -512,6 +512,17 @@ int aeon_calibrate_mfma_mix(int valu_per_mfma, int lds_reads_per_16, int iterati
 int aeon_calibrate_read_stream(const void* d_buffer, size_t bytes, int workgroups,
                                uint32_t* d_sink, size_t sink_words, void* stream);
 
+/* Launches `workgroups` workgroups of four waves that each issue `iterations` rounds of eight
+ * 16-byte-per-lane LDS reads of a 1 KiB fragment, every read waited for, the lanes addressing the
+ * fragment by `pattern`: 0 = their own order (linear), 1 = the matrix instruction's lanes reading
+ * a fragment stored position-major (16-byte unit 4 n + chunk for n = lane % 16, chunk = lane / 16),
+ * 2 = the same with each position's four pieces rotated by n / 2 (unit 4 n + (chunk + n / 2) % 4:
+ * what the grouped kernel reads), 3 = rotated by n / 4. Writes one word per thread to d_sink
+ * (>= workgroups*256 words); *wave_reads (host, optional) receives the number of wave-wide reads
+ * of the launch. Timed by the caller, it shows which orders are free of bank conflicts. */
+int aeon_calibrate_lds_read(int pattern, int iterations, int workgroups, uint32_t* d_sink,
+                            size_t sink_words, double* wave_reads, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

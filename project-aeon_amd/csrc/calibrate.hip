@@ -117,9 +117,63 @@ __global__ __launch_bounds__(256) void calibrate_read_kernel(const u32x4_t* __re
     sink[blockIdx.x * 256 + threadIdx.x] = fold[0] ^ fold[1] ^ fold[2] ^ fold[3];
 }
 
+// Fourth aid: what a 16-byte LDS read per lane costs when the lanes address a 1 KiB fragment in
+// an order other than their own. PATTERN 0: unit = lane (linear); 1: unit = 4 n + chunk, the
+// matrix instruction's lanes (n = lane % 16, chunk = lane / 16) reading a fragment stored
+// position-major; 2: unit = 4 n + (chunk + n / 2) % 4, the same with each position's four pieces
+// rotated by n / 2 (what the grouped kernel reads); 3: rotated by n / 4.
+template <int PATTERN>
+__global__ __launch_bounds__(256) void calibrate_lds_kernel(uint32_t* sink, int iterations) {
+    __shared__ u32x4_t lds[8 * 64];
+    for (int i = threadIdx.x; i < 8 * 64; i += 256) lds[i] = u32x4_t{static_cast<uint32_t>(i), 1u, 2u, 3u};
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const int n = lane & 15, chunk = lane >> 4;
+    const int unit = PATTERN == 0   ? lane
+                     : PATTERN == 1 ? 4 * n + chunk
+                     : PATTERN == 2 ? 4 * n + ((chunk + (n >> 1)) & 3)
+                                    : 4 * n + ((chunk + (n >> 2)) & 3);
+    u32x4_t fold = {0u, 0u, 0u, 0u};
+    for (int it = 0; it < iterations; ++it) {
+#pragma unroll
+        for (int f = 0; f < 8; ++f) {
+            u32x4_t t;
+            // volatile: every read is issued, and waited for before the next
+            asm volatile("ds_read_b128 %0, %1 offset:%2\n\ts_waitcnt lgkmcnt(0)"
+                         : "=v"(t)
+                         : "v"(static_cast<uint32_t>(unit * 16)), "n"(f * 1024)
+                         : "memory");
+            fold ^= t;
+        }
+    }
+    sink[blockIdx.x * 256 + threadIdx.x] = fold[0] ^ fold[1] ^ fold[2] ^ fold[3];
+}
+
 }  // namespace aeon355
 
 using namespace aeon355;
+
+extern "C" int aeon_calibrate_lds_read(int pattern, int iterations, int workgroups, uint32_t* d_sink,
+                                       size_t sink_words, double* wave_reads, void* stream) {
+    const char* who = "aeon_calibrate_lds_read";
+    AEON_REQUIRE(d_sink != nullptr && iterations > 0 && workgroups > 0 && pattern >= 0 && pattern <= 3,
+                 AEON_ERR_INVALID_ARGUMENT, "%s: bad arguments (pattern=%d iterations=%d workgroups=%d)",
+                 who, pattern, iterations, workgroups);
+    AEON_REQUIRE(sink_words >= static_cast<size_t>(workgroups) * 256, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: the sink holds %zu words, %zu needed", who, sink_words,
+                 static_cast<size_t>(workgroups) * 256);
+    hipStream_t s = as_stream(stream);
+    switch (pattern) {
+        case 0: calibrate_lds_kernel<0><<<workgroups, 256, 0, s>>>(d_sink, iterations); break;
+        case 1: calibrate_lds_kernel<1><<<workgroups, 256, 0, s>>>(d_sink, iterations); break;
+        case 2: calibrate_lds_kernel<2><<<workgroups, 256, 0, s>>>(d_sink, iterations); break;
+        default: calibrate_lds_kernel<3><<<workgroups, 256, 0, s>>>(d_sink, iterations); break;
+    }
+    AEON_LAUNCH_CHECK();
+    // four waves a workgroup, eight reads a round
+    if (wave_reads != nullptr) *wave_reads = static_cast<double>(workgroups) * 4.0 * iterations * 8.0;
+    return AEON_OK;
+}
 
 extern "C" int aeon_calibrate_read_stream(const void* d_buffer, size_t bytes, int workgroups,
                                           uint32_t* d_sink, size_t sink_words, void* stream) {

@@ -70,6 +70,8 @@ def test_argument_errors_without_device_work():
                   8, 4, None)
     with pytest.raises(ValueError, match="the sink holds"):
         capi.call("aeon_calibrate_mfma_f16", 1, 10, 4, one, C.c_size_t(512), None, None)
+    with pytest.raises(ValueError, match="bad arguments"):
+        capi.call("aeon_calibrate_lds_read", 7, 10, 4, one, C.c_size_t(1024), None, None)
     from project_aeon_amd import moe
     cfg = moe.MoeLayerStruct(7168, 2048, 256, 8, 1, 7.0, 1, 1.0, 1, None, None, 16, 128)
     assert capi.lib().aeon_moe_layer_workspace_bytes(C.byref(cfg), 64) > 0
