@@ -58,6 +58,24 @@ def measured_traffic(batch, experts, bias_scale=1.0):
                        t["write_size_kib_per_dispatch"] * t["write_scale"]))
 
 
+class _Calibration:
+    """ctypes view of calibration/libaeon_calibrate.so: the measurement aids behind the
+    --calibrate-* legs (calibration/aeon_calibrate.h). They are not part of the product library."""
+
+    def __init__(self):
+        path = os.path.join(ROOT, "calibration", "libaeon_calibrate.so")
+        if not os.path.exists(path):
+            raise RuntimeError("calibration/libaeon_calibrate.so is not built: run "
+                               "__graft_entry__.build() or make -C calibration")
+        self.lib = C.CDLL(path)
+        self.lib.aeon_calibrate_last_error.restype = C.c_char_p
+
+    def call(self, name, *args):
+        rc = getattr(self.lib, name)(*args)
+        if rc != 0:
+            raise (ValueError if rc == 1 else RuntimeError)(self.lib.aeon_calibrate_last_error().decode())
+
+
 def settle(fn, torch, seconds=0.3):
     """Untimed: keeps the GPU busy with the workload itself until its clocks have left the idle
     state (a launch after a host-side pause runs about 10 % slow for the first tens of
@@ -74,6 +92,7 @@ def settle(fn, torch, seconds=0.3):
 def calibrate_read(capi, torch):
     """What a read-only stream sustains from HBM on this GPU: 1.5 GiB (the size of a decode
     step's gate/up weights at batch 64) read once by 1024..12288 workgroups."""
+    cal = _Calibration()
     nbytes = 3 << 29
     buf = torch.randint(0, 2 ** 31 - 1, (nbytes // 4,), dtype=torch.int32, device="cuda")
     out = {"bytes": nbytes, "hbm_peak_gbps": HBM_PEAK_GBPS}
@@ -81,7 +100,7 @@ def calibrate_read(capi, torch):
         sink = torch.empty(wgs * 256, dtype=torch.int32, device="cuda")
 
         def launch(i=0):
-            capi.call("aeon_calibrate_read_stream", capi.vp(buf), C.c_size_t(nbytes), wgs,
+            cal.call("aeon_calibrate_read_stream", capi.vp(buf), C.c_size_t(nbytes), wgs,
                       capi.vp(sink), C.c_size_t(sink.numel()), None)
         settle(launch, torch, seconds=0.3)
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -98,6 +117,7 @@ def calibrate_lds(capi, torch):
     """Cost of a 16-byte-per-lane LDS read of a 1 KiB fragment by the order the lanes address it
     in (nanoseconds per wave-wide read and CU, every read waited for): their own order, the matrix
     instruction's lanes on a position-major fragment, and the same with the pieces rotated."""
+    cal = _Calibration()
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     wgs = cus * 4
     sink = torch.empty(wgs * 256, dtype=torch.int32, device="cuda")
@@ -107,7 +127,7 @@ def calibrate_lds(capi, torch):
         reads = C.c_double(0.0)
 
         def launch(i=0):
-            capi.call("aeon_calibrate_lds_read", pattern, 2000, wgs, capi.vp(sink), C.c_size_t(sink.numel()),
+            cal.call("aeon_calibrate_lds_read", pattern, 2000, wgs, capi.vp(sink), C.c_size_t(sink.numel()),
                       C.byref(reads), None)
         settle(launch, torch, seconds=0.2)
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -124,6 +144,7 @@ def calibrate_mfma(capi, torch):
     """Sustained fp16 matrix-pipe rates of this GPU, for reading the prefill figure: the
     library's register-resident MFMA loop (two waves per SIMD) with constant and with random
     operands, and torch's fp16 matmul (the vendor GEMM) at 8192^3."""
+    cal = _Calibration()
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     wgs = cus * 2
     sink = torch.empty(wgs * 256, dtype=torch.float32, device="cuda")
@@ -132,7 +153,7 @@ def calibrate_mfma(capi, torch):
         flop = C.c_double(0.0)
 
         def launch(i=0):
-            capi.call("aeon_calibrate_mfma_f16", rnd, 40000, wgs, capi.vp(sink),
+            cal.call("aeon_calibrate_mfma_f16", rnd, 40000, wgs, capi.vp(sink),
                       C.c_size_t(sink.numel()), C.byref(flop), None)
         settle(launch, torch, seconds=0.3)
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -142,23 +163,31 @@ def calibrate_mfma(capi, torch):
         b.record()
         torch.cuda.synchronize()
         out["mfma_loop_tflops_" + name] = round(flop.value * 5 / (a.elapsed_time(b) * 1e-3) / 1e12, 1)
-    # the same loop with the grouped GEMM's companion instructions between the MFMAs
+    # the same loop with the grouped GEMM's companion instructions between the MFMAs: per
+    # 16-cycle matrix slot V unpack-style VALU instructions, L LDS reads per 16 slots, both MFMA
+    # shapes (16x16x32: one per slot; 32x32x16: one per two slots), two waves per SIMD and one
     mix = {}
-    for valu, lds in ((0, 0), (1, 0), (2, 0), (3, 0), (4, 0), (1, 4), (2, 4), (3, 4), (1, 8), (3, 8)):
-        flop = C.c_double(0.0)
+    two_waves = ((0, 0), (1, 0), (2, 0), (3, 0), (4, 0), (1, 4), (2, 4), (3, 4), (1, 8), (3, 8))
+    one_wave = ((0, 0), (1, 4), (2, 4), (2, 2))
+    for waves, pairs in ((2, two_waves), (1, one_wave)):
+        for shape in (16, 32):
+            for valu, lds in pairs:
+                flop = C.c_double(0.0)
+                n_wgs = cus * waves
+                mix_sink = sink[:n_wgs * 256]
 
-        def launch(i=0):
-            capi.call("aeon_calibrate_mfma_mix", valu, lds, 20000, wgs, capi.vp(sink),
-                      C.c_size_t(sink.numel()), C.byref(flop), None)
-        settle(launch, torch, seconds=0.3)
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        for _ in range(5):
-            launch()
-        b.record()
-        torch.cuda.synchronize()
-        mix["%d_valu_%d_lds_reads_per_16" % (valu, lds)] = round(
-            flop.value * 5 / (a.elapsed_time(b) * 1e-3) / 1e12, 1)
+                def launch(i=0):
+                    cal.call("aeon_calibrate_mfma_mix", shape, valu, lds, waves, 10000, n_wgs,
+                             capi.vp(mix_sink), C.c_size_t(mix_sink.numel()), C.byref(flop), None)
+                settle(launch, torch, seconds=0.2)
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                for _ in range(5):
+                    launch()
+                b.record()
+                torch.cuda.synchronize()
+                mix["mfma%d_%dwave_%d_valu_%d_lds_reads_per_16" % (shape, waves, valu, lds)] = round(
+                    flop.value * 5 / (a.elapsed_time(b) * 1e-3) / 1e12, 1)
     out["mfma_mix_tflops_random_operands"] = mix
     n = 8192
     x = torch.randn(n, n, device="cuda", dtype=torch.float16)

@@ -292,7 +292,12 @@ typedef struct {
     const float* d_router_weight; /* fp32 [hidden][experts]; only aeon_moe_layer_decode reads it */
     const float* d_router_bias;   /* fp32 [experts], nullable */
     const aeon_a64_expert* d_experts;
-    int scale_group; /* columns per scale of every expert in the table: 128 (0 reads as 128) or 32 */
+    /* Columns per scale of every expert in the table, 128 or 32: the value the table's experts
+     * were packed with (aeon_a64_repack_*, aeon_resident_load_layer, V4ResidentExpertPool::
+     * scale_group()). The table itself carries no record of it and the two groupings differ in
+     * stride, so there is no default: any other value, 0 included, is refused with
+     * AEON_ERR_INVALID_ARGUMENT. */
+    int scale_group;
     /* The real model's dense fp16 pieces (all optional, NULL = absent):
      * the router gate as the checkpoint stores it, fp16 [experts][hidden], read by
      * aeon_moe_layer_decode when d_router_weight is NULL -- logits are then rounded to fp16 and
@@ -481,47 +486,6 @@ int aeon_resident_load_layer(const aeon_expert_catalog* catalog, uint32_t layer,
 int aeon_synth_matrix_swizzled(uint64_t seed, int expert, int matrix, int N, int K, int rpw,
                                int lpr, int scale_group, void* d_packed, void* d_scale,
                                void* stream);
-
-/* ------------------------------------------------------------------------------------------
- * Measurement aid (no counterpart in the reference)
- * ---------------------------------------------------------------------------------------- */
-
-/* Launches `workgroups` workgroups of four waves that each run `iterations` rounds of 16
- * independent v_mfma_f32_16x16x32_f16 out of registers, with constant (random_operands = 0) or
- * pseudo-random fp16 operands, and writes one float per thread to d_sink (>= workgroups*256
- * floats). *flop (host, optional) receives the FLOPs of the launch. Timed by the caller, it
- * gives the matrix-pipe rate this GPU sustains at the clock its power limit allows for such
- * data: the practical ceiling next to the published fp16 peak. */
-int aeon_calibrate_mfma_f16(int random_operands, int iterations, int workgroups, float* d_sink,
-                            size_t sink_floats, double* flop, void* stream);
-
-/* The same loop with random operands and, after every MFMA, `valu_per_mfma` independent VALU
- * instructions of the int4 unpack (v_and_or_b32, v_pk_add_f16), plus `lds_reads_per_16` 16-byte
- * LDS reads per 16 MFMAs. Served pairs: (0..4, 0), (1..3, 4), (1, 8), (3, 8); any other pair is an
- * AEON_ERR_INVALID_ARGUMENT. Gives the rate an instruction mix reaches with no memory wait at
- * all, which is what the grouped GEMM's window bodies are read against. */
-int aeon_calibrate_mfma_mix(int valu_per_mfma, int lds_reads_per_16, int iterations,
-                            int workgroups, float* d_sink, size_t sink_floats, double* flop,
-                            void* stream);
-
-/* Launches `workgroups` workgroups that each read their own contiguous bytes/workgroups share
- * of d_buffer once (16-byte loads, eight in flight per lane; the share must be a multiple of
- * 32 KiB) and write one folded word per thread to d_sink (>= workgroups*256 words). Timed by
- * the caller, it gives the rate a read-only stream sustains from HBM on this GPU: the practical
- * ceiling of the weight-streaming kernels next to the published bandwidth. */
-int aeon_calibrate_read_stream(const void* d_buffer, size_t bytes, int workgroups,
-                               uint32_t* d_sink, size_t sink_words, void* stream);
-
-/* Launches `workgroups` workgroups of four waves that each issue `iterations` rounds of eight
- * 16-byte-per-lane LDS reads of a 1 KiB fragment, every read waited for, the lanes addressing the
- * fragment by `pattern`: 0 = their own order (linear), 1 = the matrix instruction's lanes reading
- * a fragment stored position-major (16-byte unit 4 n + chunk for n = lane % 16, chunk = lane / 16),
- * 2 = the same with each position's four pieces rotated by n / 2 (unit 4 n + (chunk + n / 2) % 4:
- * what the grouped kernel reads), 3 = rotated by n / 4. Writes one word per thread to d_sink
- * (>= workgroups*256 words); *wave_reads (host, optional) receives the number of wave-wide reads
- * of the launch. Timed by the caller, it shows which orders are free of bank conflicts. */
-int aeon_calibrate_lds_read(int pattern, int iterations, int workgroups, uint32_t* d_sink,
-                            size_t sink_words, double* wave_reads, void* stream);
 
 #ifdef __cplusplus
 }

@@ -176,8 +176,20 @@ __global__ __launch_bounds__(256) void dense_f16_kernel(DenseArgs a) {
     }
 }
 
+static bool aligned_to(const void* p, uintptr_t bytes) {
+    return (reinterpret_cast<uintptr_t>(p) & (bytes - 1)) == 0;
+}
+
 static int launch_dense(const DenseArgs& a, int matrices, hipStream_t stream) {
     if (a.tokens <= 0) return AEON_OK;
+    // The kernel loads activations and weights 16 bytes a lane and stores four fp16 results
+    // (8 bytes) or four fp32 (16 bytes) at a time: a base that is off those boundaries (a slice
+    // of a larger tensor, say) would fault on the device instead of failing here.
+    bool bases_ok = aligned_to(a.x, 16) && (a.y32 == nullptr || aligned_to(a.y32, 16));
+    for (int m = 0; m < matrices; ++m) bases_ok = bases_ok && aligned_to(a.w[m], 16) && aligned_to(a.y[m], 8);
+    AEON_REQUIRE(bases_ok, AEON_ERR_INVALID_ARGUMENT,
+                 "dense fp16 GEMV: activations, weights and fp32 outputs must start on a 16-byte "
+                 "boundary and fp16 outputs on an 8-byte one");
     const int tiles = a.out_dim / 16;
     if (a.tokens <= 16) {
         dense_f16_kernel<1><<<dim3(tiles, matrices, 1), 256, 0, stream>>>(a);
@@ -232,6 +244,8 @@ int launch_dense_shared_expert(const void* d_x, long x_stride, int tokens, const
     if (int rc = launch_dense(gu, 2, stream)) return rc;
     // the activation is applied once, between the launches: inside the W2 launch every one of
     // its row-tile workgroups would redo it for all of the tokens' columns
+    AEON_REQUIRE(aligned_to(d_hidden, 16), AEON_ERR_INVALID_ARGUMENT,
+                 "dense shared expert: the gate, up and hidden scratch rows must start on a 16-byte boundary");
     const int units = tokens * (intermediate / 8);
     dense_swiglu_kernel<<<(units + 255) / 256, 256, 0, stream>>>(
         static_cast<const u32x4_t*>(d_gate), static_cast<const u32x4_t*>(d_up),

@@ -17,4 +17,4 @@ void set_error(const char* fmt, ...) {
 }  // namespace aeon355
 
 extern "C" const char* aeon_last_error(void) { return aeon355::g_error; }
-extern "C" int aeon_abi_version(void) { return 2; }
+extern "C" int aeon_abi_version(void) { return 3; }

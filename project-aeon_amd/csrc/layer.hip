@@ -111,8 +111,11 @@ static int check_layer(const aeon_moe_layer* L, const char* who) {
     AEON_REQUIRE(dense_given == 0 || (dense_given == 3 && !L->has_shared), AEON_ERR_INVALID_ARGUMENT,
                  "%s: a dense shared expert needs all three matrices and has_shared == 0 (the int4 "
                  "always-on expert and the dense one exclude each other)", who);
-    AEON_REQUIRE(L->scale_group == 0 || L->scale_group == 128 || L->scale_group == 32,
-                 AEON_ERR_INVALID_ARGUMENT, "%s: scale_group must be 128 (or 0) or 32, not %d", who,
+    // The table carries no record of how its scales are grouped, and the two groupings have
+    // different strides: a default here could silently disagree with the pool's default.
+    AEON_REQUIRE(L->scale_group == 128 || L->scale_group == 32, AEON_ERR_INVALID_ARGUMENT,
+                 "%s: scale_group must say how the table's experts were packed, 128 or 32 (got %d; a "
+                 "zero-initialised layer has to set it from the pool that made the table)", who,
                  L->scale_group);
     return AEON_OK;
 }

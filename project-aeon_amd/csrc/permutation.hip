@@ -119,14 +119,18 @@ __global__ __launch_bounds__(1024) void permutation_offsets_kernel(PermutationAr
     const int last_count = count - (segments - 1) * a.seg_tokens;
     const int light = segments > 0 && 2 * last_count <= a.seg_tokens ? 1 : 0;
     const int heavy = segments - light;
+    // One 64-bit scan carries three sums: positions in bits 0..23, heavy segments in 24..43,
+    // light ones from 44 up (launch_permutation refuses totals that would carry from one field
+    // into the next). Without a segment list the position count has the whole word.
     const unsigned long long packed = static_cast<unsigned long long>(count) |
                                       (static_cast<unsigned long long>(heavy) << 24) |
                                       (static_cast<unsigned long long>(light) << 44);
     const unsigned long long before = block_exclusive_scan3(packed, wave_totals, &total);
     const unsigned long long sums = total;
-    const int offset = static_cast<int>(before & 0xFFFFFFull);
+    const unsigned long long count_field = with_segments ? 0xFFFFFFull : ~0ull;
+    const int offset = static_cast<int>(before & count_field);
     if (e < lists) a.offsets[e] = offset;
-    if (e == 0) a.offsets[lists] = static_cast<int>(sums & 0xFFFFFFull);
+    if (e == 0) a.offsets[lists] = static_cast<int>(sums & count_field);
 
     if (with_segments) {
         const int heavy_base = static_cast<int>((before >> 24) & 0xFFFFFull);
@@ -216,6 +220,17 @@ __global__ __launch_bounds__(1024) void permutation_scatter_kernel(PermutationAr
 
 int launch_permutation(const PermutationArgs& args, hipStream_t stream) {
     PermutationArgs a = args;
+    if (a.seg_expert != nullptr) {
+        // the packed scan of the offsets kernel: 24 bits of positions, 20 of segments per class
+        const long long positions = static_cast<long long>(a.draws) + a.shared_tokens;
+        const long long lists = a.experts + (a.shared_tokens > 0 ? 1 : 0);
+        AEON_REQUIRE(a.seg_tokens > 0 && positions < (1ll << 24) &&
+                         positions / a.seg_tokens + lists < (1ll << 20),
+                     AEON_ERR_INVALID_ARGUMENT,
+                     "permutation with a segment list: %lld positions in segments of %d exceed the "
+                     "2^24 positions / 2^20 segments one launch orders; split the chunk",
+                     positions, a.seg_tokens);
+    }
     a.slots_reciprocal = 0;
     if (a.slots > 1 && static_cast<uint64_t>(a.draws) * a.slots < (1ull << 32)) {
         a.slots_reciprocal = static_cast<unsigned>(((1ull << 32) + a.slots - 1) / a.slots);

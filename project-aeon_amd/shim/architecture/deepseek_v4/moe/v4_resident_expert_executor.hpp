@@ -21,8 +21,14 @@ namespace aeon::core {
 
 class V4ResidentExpertExecutor final : public V4RoutedExpertExecutor {
 public:
-    // `layers[l]` describes layer l (experts resident, has_shared = 0: the layer body has
-    // already written the shared expert into moe_accum). `max_tokens` sizes the workspace.
+    // `layers[l]` describes layer l (experts resident). `max_tokens` sizes the workspace.
+    // Behind this seam the reference's layer body has already run the shared expert into
+    // moe_accum (run_layer_body_moe_shared_expert, layer/v4_layer_body_moe.hpp:216-256) before it
+    // calls accumulate_routed*, and the routed sum is added to what it finds there. The executor's
+    // copy of each layer therefore carries no shared expert of either kind: has_shared is cleared
+    // and so are the dense fp16 shared-expert matrices, which only aeon_moe_layer_decode (the
+    // whole step on the device) uses. A layer description filled for both uses can be passed as
+    // it is.
     V4ResidentExpertExecutor(std::vector<aeon_moe_layer> layers, int max_tokens, hipStream_t stream)
         : layers_(std::move(layers)), max_tokens_(max_tokens), stream_(stream) {
         if (layers_.empty() || max_tokens <= 0) {
@@ -31,6 +37,9 @@ public:
         int widest_top_k = 0;
         for (aeon_moe_layer& layer : layers_) {
             layer.has_shared = 0;
+            layer.d_shared_w1_f16 = nullptr;
+            layer.d_shared_w3_f16 = nullptr;
+            layer.d_shared_w2_f16 = nullptr;
             widest_top_k = std::max(widest_top_k, layer.top_k);
             workspace_bytes_ = std::max(workspace_bytes_, aeon_moe_layer_workspace_bytes(&layer, max_tokens));
         }

@@ -67,6 +67,18 @@ public:
     size_t resident_bytes() const { return slot_bytes_ * experts_per_layer_ * layers_; }
     // What aeon_moe_layer::scale_group has to say for a layer over this pool's tables.
     int scale_group() const { return scale_group_; }
+    // A layer description over this pool's table of layer l with the geometry and the scale
+    // grouping the pool was built with filled in, so the two cannot disagree; the caller adds
+    // the routing fields (top_k, score kind, gate, bias, ...).
+    aeon_moe_layer describe_layer(uint32_t layer) const {
+        aeon_moe_layer L{};
+        L.hidden = hidden_;
+        L.intermediate = intermediate_;
+        L.experts = static_cast<int>(experts_per_layer_);
+        L.d_experts = table(layer);
+        L.scale_group = scale_group_;
+        return L;
+    }
     // Device table of layer l: experts_per_layer() entries.
     const aeon_a64_expert* table(uint32_t layer) const {
         if (layer >= layers_) throw std::out_of_range("V4ResidentExpertPool: layer past the catalog");

@@ -114,8 +114,22 @@ int main() {
     half* d_x = to_device(x);
     core::V4ResidentExpertExecutor resident(layers, 16, nullptr);
     DirectPayloadExecutor direct(experts);
+    // A layer description filled for the whole-step entry point as well carries the dense fp16
+    // shared expert. Behind this seam the caller's layer body has already run it into moe_accum,
+    // so the executor must add the routed sum to what it finds and never run (or overwrite with)
+    // the dense expert: same bits as the executor built without those pointers.
+    void* d_dense = nullptr;
+    GATE_HIP(hipMalloc(&d_dense, sizeof(half) * static_cast<size_t>(kHidden) * kIntermediate));
+    GATE_HIP(hipMemset(d_dense, 0x3C, sizeof(half) * static_cast<size_t>(kHidden) * kIntermediate));
+    std::vector<aeon_moe_layer> layers_with_dense = layers;
+    for (aeon_moe_layer& layer : layers_with_dense) {
+        layer.d_shared_w1_f16 = d_dense;
+        layer.d_shared_w3_f16 = d_dense;
+        layer.d_shared_w2_f16 = d_dense;
+    }
+    core::V4ResidentExpertExecutor resident_dense(layers_with_dense, 16, nullptr);
 
-    double worst = 0, peak = 0, probe = 0, batch_delta = 0;
+    double worst = 0, peak = 0, probe = 0, batch_delta = 0, dense_delta = 0;
     for (int l = 0; l < kLayers; ++l) {
         std::vector<std::vector<int32_t>> ids(kTokens);
         std::vector<std::vector<float>> weights(kTokens);
@@ -134,7 +148,12 @@ int main() {
         half* d_out_dir = to_device(shared);
         half* d_out_probe = to_device(shared);
         half* d_out_batch = to_device(shared);
+        half* d_out_dense = to_device(shared);
+        half* d_out_dense_batch = to_device(shared);
         for (int t = 0; t < kTokens; ++t) {
+            resident_dense.on_routing_ready(l, 40 + t, ids[t], weights[t]);
+            resident_dense.accumulate_routed(l, 40 + t, d_x + static_cast<size_t>(t) * kHidden, d_w + t * kSlots,
+                                             d_out_dense + static_cast<size_t>(t) * kHidden);
             resident.on_routing_ready(l, 40 + t, ids[t], weights[t]);
             resident.accumulate_routed(l, 40 + t, d_x + static_cast<size_t>(t) * kHidden, d_w + t * kSlots,
                                        d_out_res + static_cast<size_t>(t) * kHidden);
@@ -151,6 +170,9 @@ int main() {
         resident.on_routing_ready_batch(l, 100, ids, weights);
         resident.accumulate_routed_batch(l, 100, kTokens, d_x, kHidden, d_ids, kSlots, d_w, kSlots, d_out_batch,
                                          kHidden);
+        resident_dense.on_routing_ready_batch(l, 100, ids, weights);
+        resident_dense.accumulate_routed_batch(l, 100, kTokens, d_x, kHidden, d_ids, kSlots, d_w, kSlots,
+                                               d_out_dense_batch, kHidden);
         GATE_HIP(hipGetLastError());
         GATE_HIP(hipDeviceSynchronize());
         const size_t n = static_cast<size_t>(kTokens) * kHidden;
@@ -160,6 +182,8 @@ int main() {
         peak = std::fmax(peak, p);
         probe = std::fmax(probe, max_abs_over_peak(d, to_host(d_out_probe, n), nullptr));
         batch_delta = std::fmax(batch_delta, max_abs_over_peak(r, to_host(d_out_batch, n), nullptr));
+        dense_delta = std::fmax(dense_delta, max_abs_over_peak(r, to_host(d_out_dense, n), nullptr));
+        dense_delta = std::fmax(dense_delta, max_abs_over_peak(r, to_host(d_out_dense_batch, n), nullptr));
     }
     std::printf("  resident vs direct payload: %.3e of peak %.3e; wrong-expert probe %.3e; chunk vs per-token %.3e\n",
                 worst, peak, probe, batch_delta);
@@ -167,6 +191,8 @@ int main() {
     expect(worst <= 2e-3, "resident executor within 2e-3 of peak of the direct-payload control");
     expect(probe > 50 * worst && probe > 1e-2, "a wrong expert in one slot changes the result materially");
     expect(batch_delta == 0.0, "chunk form bit-identical to the per-token form");
+    expect(dense_delta == 0.0, "dense shared-expert pointers in the layer description change nothing behind the seam: "
+                               "moe_accum is added to, not overwritten");
 
     bool logic = false, range = false, shape = false;
     try {

@@ -23,7 +23,30 @@ def test_every_declared_symbol_is_exported():
     assert len(names) >= 30
     missing = [n for n in names if not hasattr(lib, n)]
     assert not missing, missing
-    assert lib.aeon_abi_version() == 2
+    assert lib.aeon_abi_version() == 3
+
+
+def test_measurement_aids_live_outside_the_product_library():
+    """The benchmark's calibration kernels have a library and a header of their own: the product
+    library exports none of them, calibration/libaeon_calibrate.so exports everything its header
+    declares, and its argument checks fire before any launch."""
+    lib = capi.lib()
+    text = open(os.path.join(ROOT, "calibration", "aeon_calibrate.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(aeon_calibrate_[a-z0-9_]+)\s*\(", text)))
+    assert len(names) == 5, names
+    assert not [n for n in names if hasattr(lib, n)]
+    path = os.path.join(ROOT, "calibration", "libaeon_calibrate.so")
+    assert os.path.exists(path), "calibration/libaeon_calibrate.so is not built (make -C calibration)"
+    cal = C.CDLL(path)
+    assert not [n for n in names if not hasattr(cal, n)]
+    cal.aeon_calibrate_last_error.restype = C.c_char_p
+    one = C.c_void_p(16)   # never dereferenced
+    assert cal.aeon_calibrate_mfma_f16(1, 10, 4, one, C.c_size_t(512), None, None) == 1
+    assert b"the sink holds" in cal.aeon_calibrate_last_error()
+    assert cal.aeon_calibrate_lds_read(7, 10, 4, one, C.c_size_t(1024), None, None) == 1
+    assert cal.aeon_calibrate_mfma_mix(16, 7, 0, 2, 10, 4, one, C.c_size_t(1024), None, None) == 1
+    assert b"no kernel for" in cal.aeon_calibrate_last_error()
 
 
 def test_header_compiles_as_c():
@@ -68,16 +91,31 @@ def test_argument_errors_without_device_work():
     with pytest.raises(ValueError, match="null weight pointer"):
         capi.call("aeon_moe_fused_w2_accum", one, C.byref(w2), one, None, one, one, 2, 4096, 2048,
                   8, 4, None)
-    with pytest.raises(ValueError, match="the sink holds"):
-        capi.call("aeon_calibrate_mfma_f16", 1, 10, 4, one, C.c_size_t(512), None, None)
-    with pytest.raises(ValueError, match="bad arguments"):
-        capi.call("aeon_calibrate_lds_read", 7, 10, 4, one, C.c_size_t(1024), None, None)
     from project_aeon_amd import moe
     cfg = moe.MoeLayerStruct(7168, 2048, 256, 8, 1, 7.0, 1, 1.0, 1, None, None, 16, 128)
     assert capi.lib().aeon_moe_layer_workspace_bytes(C.byref(cfg), 64) > 0
     assert capi.lib().aeon_moe_layer_workspace_bytes(C.byref(cfg), 1 << 28) == 0
     with pytest.raises(ValueError, match="32-bit positions"):
         capi.call("aeon_moe_layer_routed", C.byref(cfg), one, 7168, 1 << 28, one, one, one, 7168, one,
+                  C.c_size_t(1 << 40), None)
+    # the dense fp16 kernels load 16 bytes a lane: a misaligned base is refused on the host
+    big, odd = C.c_void_p(1 << 20), C.c_void_p((1 << 20) + 2)
+    with pytest.raises(ValueError, match="16-byte boundary"):
+        capi.call("aeon_dense_gemv_f16", odd, 256, big, big, 64, 1, 256, 64, None)
+    with pytest.raises(ValueError, match="16-byte boundary"):
+        capi.call("aeon_dense_gemv_f16", big, 256, odd, big, 64, 1, 256, 64, None)
+    with pytest.raises(ValueError, match="8-byte one"):
+        capi.call("aeon_dense_gemv_f16", big, 256, big, odd, 64, 1, 256, 64, None)
+    with pytest.raises(ValueError, match="16-byte boundary"):
+        capi.call("aeon_router_logits_f16", big, 256, odd, big, big, 1, 256, 64, None)
+    with pytest.raises(ValueError, match="16-byte boundary"):
+        capi.call("aeon_dense_shared_expert_f16", big, 256, 1, big, odd, big, big, big, big, big, 256,
+                  256, 128, C.c_float(7.0), None)
+    # the expert table carries no record of its scale grouping: a layer that leaves it at zero
+    # is refused rather than read with a default that may not be the pool's
+    unset = moe.MoeLayerStruct(7168, 2048, 256, 8, 1, 7.0, 1, 1.0, 1, None, None, 16, 0)
+    with pytest.raises(ValueError, match="scale_group must say"):
+        capi.call("aeon_moe_layer_routed", C.byref(unset), one, 7168, 4, one, one, one, 7168, one,
                   C.c_size_t(1 << 40), None)
     assert capi.lib().aeon_last_error() != b""
 
