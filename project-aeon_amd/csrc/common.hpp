@@ -142,10 +142,9 @@ __device__ __forceinline__ float dot2(half2_t a, half2_t b, float c) {
     return __builtin_amdgcn_fdot2(a, b, c, false);
 }
 
-// dot of the 8 weights of one word with 8 activations (a uint4 = 8 halves), fp32 accumulate.
-__device__ __forceinline__ float dot8(uint32_t w, const uint4& x, float acc) {
-    half2_t p[4];
-    unpack8(w, p);
+// dot of the 8 weights of one word (already unpacked) with 8 activations (a uint4 = 8 halves),
+// fp32 accumulate.
+__device__ __forceinline__ float dot8(const half2_t p[4], const uint4& x, float acc) {
     Word2Half x0, x1, x2, x3;
     x0.u = x.x; x1.u = x.y; x2.u = x.z; x3.u = x.w;
     acc = dot2(p[0], x0.h, acc);
@@ -153,6 +152,13 @@ __device__ __forceinline__ float dot8(uint32_t w, const uint4& x, float acc) {
     acc = dot2(p[2], x2.h, acc);
     acc = dot2(p[3], x3.h, acc);
     return acc;
+}
+
+// the same from the packed word
+__device__ __forceinline__ float dot8(uint32_t w, const uint4& x, float acc) {
+    half2_t p[4];
+    unpack8(w, p);
+    return dot8(p, x, acc);
 }
 
 __device__ __forceinline__ float half_bits_to_float(uint16_t bits) {

@@ -89,33 +89,40 @@ __global__ __launch_bounds__(WK * 64) void a64_gemv_kernel(GemvArgs a) {
         for (int j = 0; j < kGemvPrefetch; ++j) {
             const int g = g0 + j * WK;
             if (g < a.groups && mine) {
+                // the tile's nibbles become fp16 once, outside the token loop: every token of the
+                // batch multiplies the same 32 weights of the lane
+                half2_t q[NMAT][4][4];
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m) {
+                    unpack8(wq[m][j].x, q[m][0]);
+                    unpack8(wq[m][j].y, q[m][1]);
+                    unpack8(wq[m][j].z, q[m][2]);
+                    unpack8(wq[m][j].w, q[m][3]);
+                }
 #pragma unroll
                 for (int t = 0; t < TOK; ++t) {
                     if (t < a.tokens) {
                         const uint16_t* xp = a.x + t * a.x_stride + g * 128 + chunk * 8;
-                        const uint4 x0 = *reinterpret_cast<const uint4*>(xp);
-                        const uint4 x1 = *reinterpret_cast<const uint4*>(xp + 32);
-                        const uint4 x2 = *reinterpret_cast<const uint4*>(xp + 64);
-                        const uint4 x3 = *reinterpret_cast<const uint4*>(xp + 96);
+                        uint4 x[4];
+                        x[0] = *reinterpret_cast<const uint4*>(xp);
+                        x[1] = *reinterpret_cast<const uint4*>(xp + 32);
+                        x[2] = *reinterpret_cast<const uint4*>(xp + 64);
+                        x[3] = *reinterpret_cast<const uint4*>(xp + 96);
 #pragma unroll
                         for (int m = 0; m < NMAT; ++m) {
                             if (SG == 4) {
                                 // word s of the lane holds columns of 32-column group s only
                                 const uint2 s4 = sc[m][j];
-                                acc[m][t] += half_bits_to_float(static_cast<uint16_t>(s4.x & 0xFFFFu)) *
-                                             dot8(wq[m][j].x, x0, 0.0f);
-                                acc[m][t] += half_bits_to_float(static_cast<uint16_t>(s4.x >> 16)) *
-                                             dot8(wq[m][j].y, x1, 0.0f);
-                                acc[m][t] += half_bits_to_float(static_cast<uint16_t>(s4.y & 0xFFFFu)) *
-                                             dot8(wq[m][j].z, x2, 0.0f);
-                                acc[m][t] += half_bits_to_float(static_cast<uint16_t>(s4.y >> 16)) *
-                                             dot8(wq[m][j].w, x3, 0.0f);
+                                const uint16_t step_scale[4] = {
+                                    static_cast<uint16_t>(s4.x & 0xFFFFu), static_cast<uint16_t>(s4.x >> 16),
+                                    static_cast<uint16_t>(s4.y & 0xFFFFu), static_cast<uint16_t>(s4.y >> 16)};
+#pragma unroll
+                                for (int st = 0; st < 4; ++st)
+                                    acc[m][t] += half_bits_to_float(step_scale[st]) * dot8(q[m][st], x[st], 0.0f);
                             } else {
                                 float d = 0.0f;
-                                d = dot8(wq[m][j].x, x0, d);
-                                d = dot8(wq[m][j].y, x1, d);
-                                d = dot8(wq[m][j].z, x2, d);
-                                d = dot8(wq[m][j].w, x3, d);
+#pragma unroll
+                                for (int st = 0; st < 4; ++st) d = dot8(q[m][st], x[st], d);
                                 acc[m][t] += half_bits_to_float(static_cast<uint16_t>(sc[m][j].x)) * d;
                             }
                         }
@@ -164,7 +171,7 @@ __global__ __launch_bounds__(WK * 64) void a64_gemv_kernel(GemvArgs a) {
 template <int NMAT, int TOK, int SG>
 static int launch_gemv_wk_sg(const GemvArgs& a, int wk, hipStream_t stream) {
     const int tiles = a.N / 16;
-    if (wk >= 16 && tiles < 256) {
+    if (wk >= 16 && tiles < 256 && TOK < 8) {
         a64_gemv_kernel<NMAT, TOK, 16, SG, true><<<dim3(2 * tiles), 16 * 64, 0, stream>>>(a);
     } else if (wk >= 16) {
         a64_gemv_kernel<NMAT, TOK, 16, SG, false><<<dim3(tiles), 16 * 64, 0, stream>>>(a);
@@ -192,7 +199,7 @@ static int launch_gemv(const GemvArgs& a, hipStream_t stream) {
     if (a.tokens == 1) return launch_gemv_wk<NMAT, 1>(a, wk, stream);
     if (a.tokens == 2) return launch_gemv_wk<NMAT, 2>(a, wk, stream);
     if (a.tokens <= 4) return launch_gemv_wk<NMAT, 4>(a, wk, stream);
-    return launch_gemv_wk<NMAT, 8>(a, wk > 8 ? 8 : wk, stream);
+    return launch_gemv_wk<NMAT, 8>(a, wk, stream);
 }
 
 static int check_a64_shape(int N, int K, int scale_group, const char* who) {

@@ -4,6 +4,7 @@ Tolerance: max relative error 1e-2 (denominator floored at 1e-3 of the peak), th
 fp32-accumulate outputs; the reference's own GEMV gate allows 0.05 absolute
 (tests/test_w4a16_swizzled_gemv.cpp:122)."""
 import ctypes as C
+import os
 
 import numpy as np
 import pytest
@@ -288,22 +289,33 @@ def test_config1_one_expert_decode(orc, tokens, use_mfma, scale_group):
 
 
 def test_mfma_calibration_loop_runs_and_counts_its_flops():
-    """The measurement aid: constant operands of 1.0 make every accumulator entry iterations*32,
-    so the sink is checkable in closed form; random operands only have to stay finite."""
+    """The benchmark's measurement aid (calibration/libaeon_calibrate.so, not the product library):
+    constant operands of 1.0 make every accumulator entry iterations*32, so the sink is checkable
+    in closed form; random operands and the instruction-mix loop only have to stay finite."""
     torch, _, capi = _setup()
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "calibration",
+                        "libaeon_calibrate.so")
+    assert os.path.exists(path), "calibration/libaeon_calibrate.so is not built (make -C calibration)"
+    cal = C.CDLL(path)
     wgs, iters = 8, 50
     sink = torch.zeros(wgs * 256, dtype=torch.float32, device="cuda")
     flop = C.c_double(0.0)
-    capi.call("aeon_calibrate_mfma_f16", 0, iters, wgs, capi.vp(sink), C.c_size_t(sink.numel()),
-              C.byref(flop), None)
+    assert cal.aeon_calibrate_mfma_f16(0, iters, wgs, capi.vp(sink), C.c_size_t(sink.numel()),
+                                       C.byref(flop), None) == 0
     torch.cuda.synchronize()
     assert flop.value == wgs * 4 * iters * 16 * 16384.0
     # 16 tiles x 4 entries per lane, each the sum of `iters` MFMAs of 32 products of 1.0
     assert torch.all(sink == 16 * 4 * iters * 32.0)
-    capi.call("aeon_calibrate_mfma_f16", 1, iters, wgs, capi.vp(sink), C.c_size_t(sink.numel()),
-              None, None)
+    assert cal.aeon_calibrate_mfma_f16(1, iters, wgs, capi.vp(sink), C.c_size_t(sink.numel()),
+                                       None, None) == 0
     torch.cuda.synchronize()
     assert torch.isfinite(sink).all()
+    for shape, waves in ((16, 2), (32, 2), (16, 1)):
+        assert cal.aeon_calibrate_mfma_mix(shape, 2, 4, waves, iters, wgs, capi.vp(sink),
+                                           C.c_size_t(sink.numel()), C.byref(flop), None) == 0
+        torch.cuda.synchronize()
+        assert flop.value == wgs * 4 * iters * 32 * 16384.0
+        assert torch.isfinite(sink).all()
 
 
 def test_swizzled_grouped_windows_against_oracle(orc):
