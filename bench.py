@@ -659,7 +659,6 @@ def run_other_configs(pool, layer, moe, capi, synth, torch, np, H, I, E, K_TOP, 
     rng = np.random.default_rng(SEED)
     for l in range(4):
         mixes.append(moe.HyperConnection(rng.standard_normal(24).astype(np.float32)))
-    stack = moe.LayerStack(layers, mixes)
     residual = torch.from_numpy(np.stack([synth.activations(SEED, B, H, unit=50 + j)
                                           for j in range(4)])).cuda()
     # a step over an even number of layers ends in the buffer it started from, so every timed
@@ -669,38 +668,50 @@ def run_other_configs(pool, layer, moe, capi, synth, torch, np, H, I, E, K_TOP, 
                torch.empty(B, H, dtype=torch.float16, device="cuda"),
                torch.empty(B, K_TOP, dtype=torch.int32, device="cuda"),
                torch.empty(B, K_TOP, dtype=torch.float32, device="cuda"))
-
-    def one_step(i):
-        work.copy_(residual)
-        stack.step(work, scratch)
-
-    settle(one_step, torch)
-    torch.cuda.synchronize()
-    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    reps4 = max(steps // 2, 5)
-    a.record()
-    for _ in range(reps4):
-        work.copy_(residual)
-        r = stack.step(work, scratch)
-    b.record()
-    torch.cuda.synchronize()
-    ms = a.elapsed_time(b) / reps4
-    distinct = []
-    trace = []
-    work.copy_(residual)
-    r = stack.step(work, scratch, trace)
-    for entry in trace:
-        distinct.append(int(torch.unique(entry[2]).numel()))
     be = 3 * bm
-    bytes4 = sum((d + 1) * be + H * E * 4 + B * H * 2 * 2 + B * K_TOP * 8 for d in distinct) + \
-        4 * 2 * 4 * B * H * 2
-    res["config4_stack"] = {"layers": 4, "batch": B, "ms_per_step": round(ms, 4),
-                            "us_per_token": round(ms * 1e3 / B, 3),
-                            "distinct_routed_experts_per_layer": distinct,
-                            "algorithmic_bytes": int(bytes4),
-                            "achieved_gbps": round(bytes4 / (ms * 1e-3) / 1e9, 1),
-                            "frac_of_peak": round(bytes4 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-                            "finite": bool(torch.isfinite(r.float()).all())}
+    reps4 = max(steps // 2, 5)
+
+    def run_stack(stack):
+        def one_step(i):
+            work.copy_(residual)
+            stack.step(work, scratch)
+
+        settle(one_step, torch)
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps4):
+            work.copy_(residual)
+            r = stack.step(work, scratch)
+        b.record()
+        torch.cuda.synchronize()
+        ms = a.elapsed_time(b) / reps4
+        trace = []
+        work.copy_(residual)
+        r = stack.step(work, scratch, trace)
+        distinct = [int(torch.unique(entry[3]).numel()) for entry in trace]
+        bytes4 = sum((d + 1) * be + H * E * 4 + B * H * 2 * 2 + B * K_TOP * 8 for d in distinct) + \
+            4 * 2 * 4 * B * H * 2
+        return {"layers": 4, "batch": B, "ms_per_step": round(ms, 4),
+                "us_per_token": round(ms * 1e3 / B, 3),
+                "distinct_routed_experts_per_layer": distinct,
+                "algorithmic_bytes": int(bytes4),
+                "achieved_gbps": round(bytes4 / (ms * 1e-3) / 1e9, 1),
+                "frac_of_peak": round(bytes4 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                "finite": bool(torch.isfinite(r.float()).all())}
+
+    # as BASELINE writes it: nothing normalises the residual between the layers, so its scale grows,
+    # the sigmoid scores of layers 2-4 saturate and the bias alone picks their experts
+    res["config4_stack"] = run_stack(moe.LayerStack(layers, mixes, fused=True))
+    res["config4_stack"]["launches_per_layer"] = "router logits, top-k, permutation, gate/up, down, " \
+        "reduce + post-mix + next pre-combine (one launch)"
+    res["config4_stack_three_launch_tail"] = run_stack(moe.LayerStack(layers, mixes, fused=False))
+    # the same stack with the FFN RMSNorm (seeded weight around 1) on each layer's input, where the
+    # reference's layer body has it (layer/v4_layer_body_attention.hpp:113-115): every layer then
+    # routes like the one-layer configuration
+    norm_w = [torch.from_numpy((1.0 + 0.1 * rng.standard_normal(H)).astype(np.float16)).cuda()
+              for _ in range(4)]
+    res["config4_stack_normed"] = run_stack(moe.LayerStack(layers, mixes, norm_weights=norm_w, fused=True))
     return res
 
 

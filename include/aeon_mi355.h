@@ -351,6 +351,37 @@ int aeon_moe_layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, i
 int aeon_moe_layer_decode(const aeon_moe_layer* layer, const void* d_x, int x_stride, int tokens,
                           void* d_out, int out_stride, int32_t* d_topk_ids, float* d_topk_weights,
                           void* d_workspace, size_t workspace_bytes, void* stream);
+/* The hyper-connection expansion that follows the routed experts in a layer body
+ * (run_layer_body_moe_and_post, layer/v4_layer_body_moe.hpp:259-312: experts, reduce, hc_post),
+ * for aeon_moe_layer_decode_hc_post. Streams are fp16, element (t, j, h) of a residual at
+ * t*token_stride + j*stream_stride + h; post [4] and comb [16] (comb[i*4+j]) per token
+ * (mix_per_token 1) or shared by all tokens (0); input and output residual must not alias.
+ * d_next_pre_mix (nullable): the NEXT layer's pre-mix ([4], next_pre_token_stride 4 = per token,
+ * 0 = shared) -- then the next layer's input, sum_j pre[j] * residual_out[t][j][h]
+ * (hc_pre_combine_kernel, kernels/hc_sinkhorn.hpp:94-147), is written to d_next_layer_input
+ * (row pitch next_input_stride elements) in the same pass. */
+typedef struct {
+    const void* d_residual_in;
+    long token_stride;
+    long stream_stride;
+    const float* d_post_mix;
+    const float* d_comb_mix;
+    int mix_per_token;
+    void* d_residual_out;
+    const float* d_next_pre_mix;
+    int next_pre_token_stride;
+    void* d_next_layer_input;
+    long next_input_stride;
+} aeon_hc_post_args;
+/* aeon_moe_layer_decode with the fixed-order reduce, aeon_hc_post and (optionally) the next
+ * layer's aeon_hc_pre_combine done by ONE launch instead of three: d_out still receives the
+ * layer output rows, hc->d_residual_out the expanded streams. Every value is rounded to fp16
+ * where it would cross a kernel boundary in the three-launch sequence, so the results are that
+ * sequence's, bit for bit. hidden % 8 == 0, out_stride % 8 == 0 and 16-byte aligned rows. */
+int aeon_moe_layer_decode_hc_post(const aeon_moe_layer* layer, const void* d_x, int x_stride,
+                                  int tokens, void* d_out, int out_stride, int32_t* d_topk_ids,
+                                  float* d_topk_weights, const aeon_hc_post_args* hc,
+                                  void* d_workspace, size_t workspace_bytes, void* stream);
 /* aeon_moe_layer_decode with no workspace argument and no allocation. It has no counterpart in
  * the reference: it is for callers that cannot allocate device memory or carry a workspace --
  * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc. The

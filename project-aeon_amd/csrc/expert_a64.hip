@@ -891,6 +891,111 @@ int launch_token_reduce(const float* contrib, int tokens, int slots, int shared_
     return AEON_OK;
 }
 
+// token_reduce_kernel followed, in the same pass, by hc_post_kernel and (optionally) the next
+// layer's hc_pre_combine_kernel: every value crosses a kernel boundary of the unfused sequence as
+// fp16, so it is rounded to fp16 at the same three points here (the reduced row, the four
+// expanded streams, the next layer's input) and the result is the unfused sequence's, bit for bit.
+__global__ __launch_bounds__(256) void token_reduce_hc_post_kernel(
+    const float* __restrict__ contrib, int slots, int shared_base, const uint16_t* initial,
+    long initial_stride, uint16_t* out, long out_stride, int hidden,
+    const int32_t* __restrict__ ids, int experts, aeon_hc_post_args hc) {
+    const int t = blockIdx.y;
+    const int i = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    if (i >= hidden) return;
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (shared_base >= 0) {
+        const float* sh = contrib + static_cast<size_t>(shared_base + t) * hidden + i;
+        const float4_t a = *reinterpret_cast<const float4_t*>(sh);
+        const float4_t b = *reinterpret_cast<const float4_t*>(sh + 4);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            acc[q] = half_bits_to_float(float_to_half_bits(a[q]));
+            acc[4 + q] = half_bits_to_float(float_to_half_bits(b[q]));
+        }
+    } else if (initial != nullptr) {
+        const half8_t v = *reinterpret_cast<const half8_t*>(initial + t * initial_stride + i);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) acc[q] = static_cast<float>(v[q]);
+    }
+    const float* c = contrib + static_cast<size_t>(t) * slots * hidden + i;
+    for (int s0 = 0; s0 < slots; s0 += 4) {
+        float4_t v[4][2];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int s = s0 + j < slots ? s0 + j : slots - 1;
+            const float4_t* row = reinterpret_cast<const float4_t*>(c + static_cast<size_t>(s) * hidden);
+            v[j][0] = stream_load(row);
+            v[j][1] = stream_load(row + 1);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (s0 + j >= slots) break;
+            if (ids != nullptr) {
+                const int e = ids[t * slots + s0 + j];
+                if (e < 0 || e >= experts) continue;
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                acc[q] += v[j][0][q];
+                acc[4 + q] += v[j][1][q];
+            }
+        }
+    }
+    half8_t y;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) y[q] = static_cast<half_t>(acc[q]);
+    *reinterpret_cast<half8_t*>(out + t * out_stride + i) = y;
+
+    const float* pm = hc.d_post_mix + static_cast<size_t>(t) * (hc.mix_per_token ? 4 : 0);
+    const float* cm = hc.d_comb_mix + static_cast<size_t>(t) * (hc.mix_per_token ? 16 : 0);
+    const uint16_t* res_in = static_cast<const uint16_t*>(hc.d_residual_in);
+    uint16_t* res_out = static_cast<uint16_t*>(hc.d_residual_out);
+    half8_t r[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        r[k] = *reinterpret_cast<const half8_t*>(res_in + t * hc.token_stride + k * hc.stream_stride + i);
+    }
+    float next[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    const float* pre = hc.d_next_pre_mix != nullptr
+                           ? hc.d_next_pre_mix + static_cast<size_t>(t) * hc.next_pre_token_stride
+                           : nullptr;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        half8_t o;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            float v = pm[j] * static_cast<float>(y[q]);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) v += cm[k * 4 + j] * static_cast<float>(r[k][q]);
+            o[q] = static_cast<half_t>(v);
+        }
+        *reinterpret_cast<half8_t*>(res_out + t * hc.token_stride + j * hc.stream_stride + i) = o;
+        if (pre != nullptr) {
+            const float pj = pre[j];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) next[q] += pj * static_cast<float>(o[q]);
+        }
+    }
+    if (pre != nullptr) {
+        half8_t x;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) x[q] = static_cast<half_t>(next[q]);
+        *reinterpret_cast<half8_t*>(static_cast<uint16_t*>(hc.d_next_layer_input) +
+                                    t * hc.next_input_stride + i) = x;
+    }
+}
+
+int launch_token_reduce_hc_post(const float* contrib, int tokens, int slots, int shared_base,
+                                const uint16_t* initial, long initial_stride, uint16_t* out,
+                                long out_stride, int hidden, const aeon_hc_post_args& hc,
+                                hipStream_t stream, const int32_t* ids, int experts) {
+    if (tokens <= 0) return AEON_OK;
+    token_reduce_hc_post_kernel<<<dim3((hidden / 8 + 255) / 256, tokens), 256, 0, stream>>>(
+        contrib, slots, shared_base, initial, initial_stride, out, out_stride, hidden, ids, experts, hc);
+    AEON_LAUNCH_CHECK();
+    return AEON_OK;
+}
+
 }  // namespace aeon355
 
 using namespace aeon355;

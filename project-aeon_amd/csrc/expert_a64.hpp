@@ -94,4 +94,14 @@ int launch_token_reduce(const float* contrib, int tokens, int slots, int shared_
                         long out_stride, int hidden, hipStream_t stream,
                         const int32_t* ids = nullptr, int experts = 0);
 
+// The same reduce with the hyper-connection expansion that follows it in a layer body applied in
+// the same pass (the argument struct is aeon_hc_post_args of the C ABI): the token's reduced row
+// is rounded to fp16 (and stored to `out`), expanded into the four residual streams, and -- when
+// the next layer's pre-mix is given -- the next layer's input is combined from the streams as
+// they were just rounded. Eight columns a thread; hidden % 8 == 0.
+int launch_token_reduce_hc_post(const float* contrib, int tokens, int slots, int shared_base,
+                                const uint16_t* initial, long initial_stride, uint16_t* out,
+                                long out_stride, int hidden, const aeon_hc_post_args& hc,
+                                hipStream_t stream, const int32_t* ids, int experts);
+
 }  // namespace aeon355

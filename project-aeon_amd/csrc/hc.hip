@@ -249,6 +249,11 @@ __global__ __launch_bounds__(256) void hc_project_kernel(
 // out[t][i] = half(x[t][i] * rsqrt(mean(x[t]^2) + eps) * weight[i]); fp32 arithmetic, fp16 in and
 // out, fp16 weight (null = the weightless form). One workgroup per token; the sum of squares is
 // combined in the same fixed order as above.
+// VEC: rows and pitches are multiples of 8 elements and 16-byte aligned, so a thread moves eight
+// values at a time and keeps its share of the row (up to kRmsHeld x 8 values) in registers
+// between the two passes; otherwise one value at a time, the row read twice.
+constexpr int kRmsHeld = 4;  // 256 threads x 8 x 4 = rows of up to 8192 stay in registers
+template <bool VEC>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict__ x, long x_stride,
                                                       const uint16_t* __restrict__ weight,
                                                       uint16_t* __restrict__ out, long out_stride,
@@ -258,9 +263,33 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict
     const int wave = threadIdx.x >> 6;
     const uint16_t* row = x + static_cast<size_t>(token) * x_stride;
     float sum_sq = 0.0f;
-    for (int i = threadIdx.x; i < dim; i += 256) {
-        const float v = half_bits_to_float(row[i]);
-        sum_sq += v * v;
+    half8_t held[kRmsHeld];
+    if (VEC) {
+#pragma unroll
+        for (int r = 0; r < kRmsHeld; ++r) {
+            const int i = (r * 256 + threadIdx.x) * 8;
+            if (i < dim) {
+                held[r] = *reinterpret_cast<const half8_t*>(row + i);
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    const float v = static_cast<float>(held[r][q]);
+                    sum_sq += v * v;
+                }
+            }
+        }
+        for (int i = (kRmsHeld * 256 + threadIdx.x) * 8; i < dim; i += 256 * 8) {
+            const half8_t v8 = *reinterpret_cast<const half8_t*>(row + i);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const float v = static_cast<float>(v8[q]);
+                sum_sq += v * v;
+            }
+        }
+    } else {
+        for (int i = threadIdx.x; i < dim; i += 256) {
+            const float v = half_bits_to_float(row[i]);
+            sum_sq += v * v;
+        }
     }
     __shared__ float partial[4];
     const float sq = wave_xor_sum(sum_sq, 63);
@@ -269,9 +298,31 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict
     const float inv_rms =
         rsqrtf((((partial[0] + partial[1]) + partial[2]) + partial[3]) / static_cast<float>(dim) + eps);
     uint16_t* dst = out + static_cast<size_t>(token) * out_stride;
-    for (int i = threadIdx.x; i < dim; i += 256) {
-        const float w = weight != nullptr ? half_bits_to_float(weight[i]) : 1.0f;
-        dst[i] = float_to_half_bits(half_bits_to_float(row[i]) * inv_rms * w);
+    if (VEC) {
+        auto scaled = [&](const half8_t& v8, int i) {
+            half8_t w8;
+            if (weight != nullptr) w8 = *reinterpret_cast<const half8_t*>(weight + i);
+            half8_t o;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const float w = weight != nullptr ? static_cast<float>(w8[q]) : 1.0f;
+                o[q] = static_cast<half_t>(static_cast<float>(v8[q]) * inv_rms * w);
+            }
+            *reinterpret_cast<half8_t*>(dst + i) = o;
+        };
+#pragma unroll
+        for (int r = 0; r < kRmsHeld; ++r) {
+            const int i = (r * 256 + threadIdx.x) * 8;
+            if (i < dim) scaled(held[r], i);
+        }
+        for (int i = (kRmsHeld * 256 + threadIdx.x) * 8; i < dim; i += 256 * 8) {
+            scaled(*reinterpret_cast<const half8_t*>(row + i), i);
+        }
+    } else {
+        for (int i = threadIdx.x; i < dim; i += 256) {
+            const float w = weight != nullptr ? half_bits_to_float(weight[i]) : 1.0f;
+            dst[i] = float_to_half_bits(half_bits_to_float(row[i]) * inv_rms * w);
+        }
     }
 }
 
@@ -306,9 +357,18 @@ extern "C" int aeon_rmsnorm(const void* d_x, long x_stride, const void* d_weight
     AEON_REQUIRE(tokens >= 0 && dim > 0 && x_stride >= dim && out_stride >= dim,
                  AEON_ERR_INVALID_ARGUMENT, "%s: bad shape or pitch (dim=%d)", who, dim);
     if (tokens == 0) return AEON_OK;
-    rmsnorm_kernel<<<tokens, 256, 0, as_stream(stream)>>>(
-        static_cast<const uint16_t*>(d_x), x_stride, static_cast<const uint16_t*>(d_weight),
-        static_cast<uint16_t*>(d_out), out_stride, dim, eps);
+    const bool vec = dim % 8 == 0 && x_stride % 8 == 0 && out_stride % 8 == 0 &&
+                     ((reinterpret_cast<uintptr_t>(d_x) | reinterpret_cast<uintptr_t>(d_out) |
+                       reinterpret_cast<uintptr_t>(d_weight)) & 15) == 0;
+    if (vec) {
+        rmsnorm_kernel<true><<<tokens, 256, 0, as_stream(stream)>>>(
+            static_cast<const uint16_t*>(d_x), x_stride, static_cast<const uint16_t*>(d_weight),
+            static_cast<uint16_t*>(d_out), out_stride, dim, eps);
+    } else {
+        rmsnorm_kernel<false><<<tokens, 256, 0, as_stream(stream)>>>(
+            static_cast<const uint16_t*>(d_x), x_stride, static_cast<const uint16_t*>(d_weight),
+            static_cast<uint16_t*>(d_out), out_stride, dim, eps);
+    }
     AEON_LAUNCH_CHECK();
     return AEON_OK;
 }

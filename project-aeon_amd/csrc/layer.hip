@@ -145,8 +145,27 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
                                int tokens, const int32_t* d_topk_ids, const float* d_topk_weights,
                                void* d_out, int out_stride, void* d_workspace,
                                size_t workspace_bytes, int stage_mask, void* stream,
-                               const char* who) {
+                               const char* who, const aeon_hc_post_args* hc = nullptr) {
     if (int rc = check_layer(layer, who)) return rc;
+    if (hc != nullptr) {
+        AEON_REQUIRE(hc->d_residual_in && hc->d_residual_out && hc->d_post_mix && hc->d_comb_mix &&
+                         hc->d_residual_in != hc->d_residual_out,
+                     AEON_ERR_INVALID_ARGUMENT, "%s: the hyper-connection expansion needs both residuals "
+                     "(not aliased), post and comb", who);
+        AEON_REQUIRE(layer->hidden % 8 == 0 && out_stride % 8 == 0 && hc->token_stride % 8 == 0 &&
+                         hc->stream_stride % 8 == 0 &&
+                         ((reinterpret_cast<uintptr_t>(d_out) | reinterpret_cast<uintptr_t>(hc->d_residual_in) |
+                           reinterpret_cast<uintptr_t>(hc->d_residual_out)) & 15) == 0,
+                     AEON_ERR_INVALID_ARGUMENT, "%s: the fused expansion moves 16 bytes at a time: rows and "
+                     "pitches must be multiples of 8 elements and 16-byte aligned", who);
+        AEON_REQUIRE(hc->d_next_pre_mix == nullptr ||
+                         (hc->d_next_layer_input != nullptr && hc->next_input_stride >= layer->hidden &&
+                          hc->next_input_stride % 8 == 0 &&
+                          (reinterpret_cast<uintptr_t>(hc->d_next_layer_input) & 15) == 0 &&
+                          (hc->next_pre_token_stride == 0 || hc->next_pre_token_stride == 4)),
+                     AEON_ERR_INVALID_ARGUMENT, "%s: bad next-layer input (pitch %ld, pre-mix stride %d)",
+                     who, hc->next_input_stride, hc->next_pre_token_stride);
+    }
     AEON_REQUIRE(d_x && d_topk_ids && d_topk_weights && d_out && d_workspace,
                  AEON_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
     AEON_REQUIRE(tokens >= 0 && x_stride >= layer->hidden && x_stride % 8 == 0 &&
@@ -292,6 +311,12 @@ static int layer_routed_stages(const aeon_moe_layer* layer, const void* d_x, int
         }
     }
     if (!(stage_mask & AEON_STAGE_REDUCE)) return AEON_OK;
+    if (hc != nullptr) {
+        return launch_token_reduce_hc_post(
+            w.contrib, tokens, layer->top_k, layer->has_shared ? draws : -1,
+            layer->has_shared ? nullptr : static_cast<const uint16_t*>(d_out), out_stride,
+            static_cast<uint16_t*>(d_out), out_stride, layer->hidden, *hc, s, d_topk_ids, layer->experts);
+    }
     return launch_token_reduce(w.contrib, tokens, layer->top_k, layer->has_shared ? draws : -1,
                                layer->has_shared ? nullptr : static_cast<const uint16_t*>(d_out),
                                out_stride, static_cast<uint16_t*>(d_out), out_stride, layer->hidden, s,
@@ -317,11 +342,10 @@ extern "C" int aeon_moe_layer_routed_stages(const aeon_moe_layer* layer, const v
                                "aeon_moe_layer_routed_stages");
 }
 
-extern "C" int aeon_moe_layer_decode(const aeon_moe_layer* layer, const void* d_x, int x_stride,
-                                     int tokens, void* d_out, int out_stride, int32_t* d_topk_ids,
-                                     float* d_topk_weights, void* d_workspace,
-                                     size_t workspace_bytes, void* stream) {
-    const char* who = "aeon_moe_layer_decode";
+static int layer_decode(const aeon_moe_layer* layer, const void* d_x, int x_stride, int tokens,
+                        void* d_out, int out_stride, int32_t* d_topk_ids, float* d_topk_weights,
+                        void* d_workspace, size_t workspace_bytes, void* stream, const char* who,
+                        const aeon_hc_post_args* hc) {
     if (int rc = check_layer(layer, who)) return rc;
     AEON_REQUIRE(layer->d_router_weight != nullptr || layer->d_router_weight_f16 != nullptr,
                  AEON_ERR_INVALID_ARGUMENT, "%s: the layer has no router weight", who);
@@ -363,8 +387,27 @@ extern "C" int aeon_moe_layer_decode(const aeon_moe_layer* layer, const void* d_
                                     layer->score_kind, s)) {
         return rc;
     }
-    return aeon_moe_layer_routed(layer, d_x, x_stride, tokens, d_topk_ids, d_topk_weights, d_out,
-                                 out_stride, d_workspace, workspace_bytes, stream);
+    return layer_routed_stages(layer, d_x, x_stride, tokens, d_topk_ids, d_topk_weights, d_out,
+                               out_stride, d_workspace, workspace_bytes, AEON_STAGE_ALL, stream, who, hc);
+}
+
+extern "C" int aeon_moe_layer_decode(const aeon_moe_layer* layer, const void* d_x, int x_stride,
+                                     int tokens, void* d_out, int out_stride, int32_t* d_topk_ids,
+                                     float* d_topk_weights, void* d_workspace,
+                                     size_t workspace_bytes, void* stream) {
+    return layer_decode(layer, d_x, x_stride, tokens, d_out, out_stride, d_topk_ids, d_topk_weights,
+                        d_workspace, workspace_bytes, stream, "aeon_moe_layer_decode", nullptr);
+}
+
+extern "C" int aeon_moe_layer_decode_hc_post(const aeon_moe_layer* layer, const void* d_x,
+                                             int x_stride, int tokens, void* d_out, int out_stride,
+                                             int32_t* d_topk_ids, float* d_topk_weights,
+                                             const aeon_hc_post_args* hc, void* d_workspace,
+                                             size_t workspace_bytes, void* stream) {
+    const char* who = "aeon_moe_layer_decode_hc_post";
+    AEON_REQUIRE(hc != nullptr, AEON_ERR_INVALID_ARGUMENT, "%s: null hyper-connection arguments", who);
+    return layer_decode(layer, d_x, x_stride, tokens, d_out, out_stride, d_topk_ids, d_topk_weights,
+                        d_workspace, workspace_bytes, stream, who, hc);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -27,6 +27,15 @@ class MoeLayerStruct(C.Structure):
                 ("d_shared_w2_f16", C.c_void_p)]
 
 
+class HcPostArgs(C.Structure):
+    """aeon_hc_post_args of the C ABI."""
+    _fields_ = [("d_residual_in", C.c_void_p), ("token_stride", C.c_long), ("stream_stride", C.c_long),
+                ("d_post_mix", C.c_void_p), ("d_comb_mix", C.c_void_p), ("mix_per_token", C.c_int),
+                ("d_residual_out", C.c_void_p), ("d_next_pre_mix", C.c_void_p),
+                ("next_pre_token_stride", C.c_int), ("d_next_layer_input", C.c_void_p),
+                ("next_input_stride", C.c_long)]
+
+
 def stream_ptr():
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
@@ -167,6 +176,31 @@ class MoeLayer:
                   C.c_size_t(ws.numel()), stream_ptr())
         return out, ids, weights
 
+    def decode_hc_post(self, x, residual_in, residual_out, hc, next_hc=None, next_x=None, out=None,
+                       ids=None, weights=None):
+        """decode() with the fixed-order reduce, the hyper-connection expansion of `hc` (post and
+        comb of a HyperConnection; residuals fp16 [4][tokens][hidden]) and, when `next_hc` is
+        given, the next layer's pre-combine into `next_x`, in one launch
+        (aeon_moe_layer_decode_hc_post). Returns (out, ids, weights)."""
+        tokens = x.shape[0]
+        ws = self._workspace(tokens)
+        k = self.cfg.top_k
+        out = self._new_out(x) if out is None else out
+        ids = torch.empty(tokens, k, dtype=torch.int32, device=x.device) if ids is None else ids
+        weights = (torch.empty(tokens, k, dtype=torch.float32, device=x.device)
+                   if weights is None else weights)
+        per_token = int(hc.post.shape[0] > 1)
+        args = HcPostArgs(residual_in.data_ptr(), residual_in.stride(1), residual_in.stride(0),
+                          hc.post.data_ptr(), hc.comb.data_ptr(), per_token, residual_out.data_ptr(),
+                          next_hc.pre.data_ptr() if next_hc is not None else None,
+                          (4 if next_hc is not None and next_hc.pre.shape[0] > 1 else 0),
+                          next_x.data_ptr() if next_hc is not None else None,
+                          next_x.stride(0) if next_hc is not None else 0)
+        capi.call("aeon_moe_layer_decode_hc_post", C.byref(self.cfg), capi.vp(x), x.stride(0), tokens,
+                  capi.vp(out), out.stride(0), capi.vp(ids), capi.vp(weights), C.byref(args),
+                  capi.vp(ws), C.c_size_t(ws.numel()), stream_ptr())
+        return out, ids, weights
+
     def routed(self, x, ids, weights, out=None):
         """The expert part only, for given routing (ids int32 / weights fp32 [tokens][top_k]).
         A layer without an always-on expert adds the routed sum to what `out` holds (the
@@ -286,31 +320,61 @@ class DynamicHyperConnection:
 
 class LayerStack:
     """BASELINE config 4: stacked MoE layers with the hyper-connection residual mix between them.
-    Per layer: x = pre-combine(residual); y = MoE(x); residual = post-mix(y, residual)."""
+    Per layer: x = pre-combine(residual); [x = RMSNorm(x) * norm_weight]; y = MoE(x);
+    residual = post-mix(y, residual). `norm_weights`: None = no norm (the configuration as
+    written); a list with one entry per layer, each a device fp16 [hidden] weight or None for the
+    weightless norm = the FFN norm the reference's layer body applies to the layer input
+    (layer/v4_layer_body_attention.hpp:113-115). `fused` runs the reduce, the post-mix and the
+    next layer's pre-combine in the expert step's last launch instead of three launches of
+    their own; same bits."""
 
-    def __init__(self, layers, mixes):
+    def __init__(self, layers, mixes, norm_weights=None, fused=True, rms_eps=1e-6):
         assert len(layers) == len(mixes)
+        assert norm_weights is None or len(norm_weights) == len(layers)
         self.layers = layers
         self.mixes = mixes
+        self.norm_weights = norm_weights
+        self.fused = fused
+        self.rms_eps = rms_eps
+
+    def _norm(self, l, x, out):
+        capi.call("aeon_rmsnorm", capi.vp(x), C.c_long(x.stride(0)), capi.vp(self.norm_weights[l]),
+                  capi.vp(out), C.c_long(out.stride(0)), x.shape[0], x.shape[1],
+                  C.c_float(self.rms_eps), stream_ptr())
+        return out
 
     def step(self, residual, scratch=None, trace=None):
         """residual fp16 [4][tokens][hidden]; returns the new residual (a different buffer).
         `scratch` = (residual-shaped buffer, x [tokens][hidden]) and optionally the layer output,
-        ids and weights buffers every layer reuses."""
+        ids and weights buffers every layer reuses. A trace entry is (residual in, the
+        pre-combined layer input, the input as the router and experts saw it (normed, if the stack
+        norms), ids, weights, layer output, residual out)."""
         streams, tokens, hidden = residual.shape
         if scratch is None:
             scratch = (torch.empty_like(residual), torch.empty(tokens, hidden, dtype=torch.float16,
                                                                device=residual.device))
         other, x = scratch[:2]
         bufs = scratch[2:] if len(scratch) > 2 else (None, None, None)
-        for layer, hc in zip(self.layers, self.mixes):
-            hc.pre_combine(residual, x)
+        normed = self.norm_weights is not None
+        if normed and getattr(self, "_x_norm", None) is None or (normed and self._x_norm.shape != x.shape):
+            self._x_norm = torch.empty_like(x)
+        last = len(self.layers) - 1
+        for l, (layer, hc) in enumerate(zip(self.layers, self.mixes)):
+            if l == 0 or not self.fused:
+                hc.pre_combine(residual, x)
+            x_in = self._norm(l, x, self._x_norm) if normed else x
+            if trace is not None:
+                x_pre, x_seen = x.clone(), x_in.clone()
             if bufs[0] is not None and not layer.cfg.has_shared:
                 bufs[0].zero_()
-            y, ids, w = layer.decode(x, *bufs)
-            hc.post_mix(y, residual, other)
+            if self.fused:
+                nxt = self.mixes[l + 1] if l < last else None
+                y, ids, w = layer.decode_hc_post(x_in, residual, other, hc, nxt, x, *bufs)
+            else:
+                y, ids, w = layer.decode(x_in, *bufs)
+                hc.post_mix(y, residual, other)
             if trace is not None:
-                trace.append((residual.clone(), x.clone(), ids.clone(), w.clone(), y.clone(),
+                trace.append((residual.clone(), x_pre, x_seen, ids.clone(), w.clone(), y.clone(),
                               other.clone()))
             residual, other = other, residual
         return residual

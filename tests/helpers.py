@@ -136,6 +136,29 @@ def rel_err(got, want, floor_fraction=1e-3):
     return float((np.abs(got - want) / denom).max())
 
 
+def error_report(got, want):
+    """A comparison read the way the reference's `compare` reports it (dsv4_oracle.hpp:96-129):
+    the largest |got-want| / max(|want|, f * peak) for four floor fractions f. f = 1.0 is the
+    largest error as a fraction of the data's peak -- what the reference's expert gates call
+    max_rel (they pass that floor, tests/test_v4_expert_oracle.cpp:86-98) and bound by 6e-3;
+    f = 1e-3 is the function's default. For the default floor the element the maximum occurs at
+    is reported too: its index, how large the wanted value there is against the peak, and the
+    error there against the peak."""
+    got = np.asarray(got, dtype=np.float64).ravel()
+    want = np.asarray(want, dtype=np.float64).ravel()
+    peak = np.abs(want).max()
+    diff = np.abs(got - want)
+    out = {"peak": float(peak)}
+    for name, f in (("rel_floor_1", 1.0), ("rel_floor_1e-1", 1e-1), ("rel_floor_1e-2", 1e-2),
+                    ("rel_floor_1e-3", 1e-3)):
+        rel = diff / np.maximum(np.abs(want), f * peak)
+        out[name] = float(rel.max())
+    at = int(rel.argmax())
+    out.update({"floor_1e-3_at": at, "want_over_peak_there": float(abs(want[at]) / peak),
+                "abs_over_peak_there": float(diff[at] / peak)})
+    return out
+
+
 def stream_ptr():
     import torch
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)

@@ -219,6 +219,28 @@ def test_expert_permutation_bit_exact(orc, T, slots, E):
         assert np.array_equal(d_wp.cpu().numpy()[:placed], wts.reshape(-1)[drw[:placed]])
 
 
+# Chained results (gate/up -> fp16 hidden -> W2 -> reduce over nine experts) against the fp64
+# oracle, printed by the full-size tests as relative errors with the denominator floored at a
+# fraction f of the peak (helpers.error_report):
+#   * f = 1: the largest error over the peak. This is what the reference's own expert gates call
+#     max_rel and bound by 6e-3; the stated tolerance of 1e-2 is read the same way. Observed
+#     4e-4 (decode kernels) and 9e-4 (grouped GEMM, which rounds every weight times its scale to
+#     fp16 once, as the reference's grouped feed does).
+#   * f = 0.1: outputs of a tenth of the peak and more are within 1e-2 of themselves.
+#   * f = 1e-2 and 1e-3 (`compare`'s default): set by outputs where nine contributions of the
+#     size of the peak cancel to a hundredth or a thousandth of it; the error there is still a
+#     few 1e-4 of the peak, which is several per cent (decode) to tens of per cent (grouped) of
+#     such an element. Printed with the element's size; not a pass criterion beyond "finite".
+PEAK_BOUND = 6e-3
+TENTH_OF_PEAK_REL_BOUND = 1e-2
+
+
+def check_chained(report):
+    assert report["rel_floor_1"] <= PEAK_BOUND, report
+    assert report["rel_floor_1e-1"] <= TENTH_OF_PEAK_REL_BOUND, report
+    assert np.isfinite(report["rel_floor_1e-3"]), report
+
+
 def _oracle_layer(orc, h, experts, x, ids, weights, shared, limit):
     """out[t] = half-rounded-shared + sum_k w_k * FFN_{id_k}(x_t), per the fixed-order combine,
     with every FFN from the fp64 oracle (hidden rounded to fp16 as the device stores it)."""
@@ -236,6 +258,26 @@ def _oracle_layer(orc, h, experts, x, ids, weights, shared, limit):
         if shared is not None:
             sh = shared.ffn(x[t:t + 1], limit, round_hidden=True)[0].astype(np.float16).astype(np.float64)
         out[t] = orc.moe_combine(contrib[t], sh)
+    return out
+
+
+def _oracle_layer_streamed(orc, make_expert, x, ids, weights, shared, limit):
+    """_oracle_layer for samples that touch many full-size experts: every expert is made when its
+    turn comes (make_expert(id)) and dropped afterwards, so only one is in host memory at a time."""
+    T, k = ids.shape
+    H = x.shape[1]
+    contrib = np.zeros((T, k, H))
+    for e in np.unique(ids):
+        rows, slots = np.nonzero(ids == e)
+        o = make_expert(int(e)).ffn(x[rows], limit, round_hidden=True)
+        for i, (t, s) in enumerate(zip(rows, slots)):
+            contrib[t, s] = float(weights[t, s]) * o[i]
+    out = np.empty((T, H))
+    sh = None
+    if shared is not None:
+        sh = shared.ffn(x, limit, round_hidden=True).astype(np.float16).astype(np.float64)
+    for t in range(T):
+        out[t] = orc.moe_combine(contrib[t], None if sh is None else sh[t])
     return out
 
 
@@ -373,13 +415,15 @@ def test_config2_full_size_sampled(orc):
         assert np.array_equal(ids[t], oi)
         assert np.abs(w[t] - ow).max() <= 1e-5
     assert 60 <= np.unique(ids).size <= 140   # the biased router concentrates the routing
-    sample = [0, 31, 63]
-    needed = sorted(set(int(e) for t in sample for e in ids[t]))
-    experts = {e: h.Expert(0, e, H, I) for e in needed}
-    shared = h.Expert(0, E, H, I)
-    want = _oracle_layer(orc, h, experts, x[sample], ids[sample], w[sample], shared, limit)
+    # eight tokens spread over the batch; the experts' payloads come back from the device
+    # generator (held to the host generator bit for bit above), one expert at a time
+    sample = [0, 9, 18, 27, 36, 45, 54, 63]
+    want = _oracle_layer_streamed(orc, lambda e: h.GeneratedExpert(0, e, H, I), x[sample], ids[sample],
+                                  w[sample], h.GeneratedExpert(0, E, H, I), limit)
     assert np.abs(want).max() > 1.0
-    assert np.abs(out[sample] - want).max() <= 6e-3 * np.abs(want).max()
+    report = h.error_report(out[sample], want)
+    print("config 2 full size, %d tokens against the oracle: %s" % (len(sample), report))
+    check_chained(report)
     again, _, _ = layer.decode(d_x)
     assert np.array_equal(again.cpu().numpy(), out)
     rev = layer.routed(d_x.flip(0).contiguous(), ids_t.flip(0).contiguous(),
@@ -654,12 +698,37 @@ def test_config3_prefill_full_size_sampled(orc):
     torch.cuda.synchronize()
     out = out_t.cpu().numpy()
     assert np.isfinite(out).all()
-    sample = [0, 777, 2047]
-    needed = sorted(set(int(e) for t in sample for e in ids[t]))
-    experts = {e: h.Expert(0, e, H, I) for e in needed}
-    shared = h.Expert(0, E, H, I)
-    want = _oracle_layer(orc, h, experts, x[sample], ids[sample], w[sample], shared, limit)
-    assert np.abs(out[sample] - want).max() <= 6e-3 * np.abs(want).max()
+    # The sample is stratified over what the grouped kernel does differently: for every window
+    # body (1, 2, 3, 4, 6 and 8 live token tiles) the first and the last position of a window of
+    # that size, two positions deep in the hottest expert's list (beyond its 1024th), and three
+    # fixed tokens. A sampled token's whole output is checked, i.e. all eight of its experts and
+    # the always-on one, whatever windows those draws fall in.
+    order = np.argsort(ids.ravel(), kind="stable")          # draws by expert, ascending draw
+    start = np.concatenate([[0], np.cumsum(counts)])
+    token_of = lambda e, rank: int(order[start[e] + rank] // k)
+    sample = {0, 123, 555, 777, 1024, 1500, 2047}
+    hottest = int(counts.argmax())
+    assert counts[hottest] > 1700
+    sample |= {token_of(hottest, 1100), token_of(hottest, 1700)}
+    classes_seen = set()
+    for live in (1, 2, 3, 4, 6, 8):
+        for e in np.argsort(-counts):
+            tail = int(counts[e]) % 128 or (128 if counts[e] else 0)
+            tiles = (tail + 15) // 16
+            body = 1 if tiles <= 1 else 2 if tiles == 2 else 3 if tiles == 3 else 4 if tiles == 4 else 6 if tiles <= 6 else 8
+            if counts[e] and body == live:
+                first_of_window = int(counts[e]) - tail
+                sample |= {token_of(int(e), first_of_window), token_of(int(e), int(counts[e]) - 1)}
+                classes_seen.add(live)
+                break
+    assert classes_seen == {1, 2, 3, 4, 6, 8}
+    sample = sorted(sample)
+    assert len(sample) >= 16
+    want = _oracle_layer_streamed(orc, lambda e: h.GeneratedExpert(0, e, H, I), x[sample], ids[sample],
+                                  w[sample], h.GeneratedExpert(0, E, H, I), limit)
+    report = h.error_report(out[sample], want)
+    print("config 3 full size, %d tokens against the oracle: %s" % (len(sample), report))
+    check_chained(report)
     dec = layer.routed(d_x[:64], d_ids[:64], d_w[:64]).cpu().numpy()
     assert np.abs(out[:64] - dec).max() <= 2e-3 * np.abs(dec).max()
     # reversed token order: same rows, reversed (per-token results do not depend on the batch)
