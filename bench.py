@@ -46,16 +46,36 @@ def matrix_bytes(n, k):
     return n * k // 2 + n * (k // SCALE_GROUP) * 2
 
 
-def measured_traffic(batch, experts, bias_scale=1.0):
-    """HBM bytes per launch of the gate/up kernel from the committed rocprofv3 --pmc runs
-    (FETCH_SIZE, WRITE_SIZE in KiB per dispatch, each scaled by what the same counter reads for a
-    plain copy of known size), or None for a workload that was not profiled."""
-    path = os.path.join(ROOT, "profiles", "traffic_config2_decode_b%d.json" % batch)
-    if experts != 256 or bias_scale != 1.0 or not os.path.exists(path):
-        return None
+def csrc_digest():
+    """A digest of the library's sources (project-aeon_amd/csrc/*.hip, *.hpp, *.cpp and the ABI
+    header): what a committed counter profile is dated by. The GPU box runs a copy of the tree
+    without its git history, so "the kernels changed since the profile was taken" is decided by
+    content, not by commit."""
+    import hashlib
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "project-aeon_amd", "csrc")
+    names = sorted(n for n in os.listdir(csrc) if n.endswith((".hip", ".hpp", ".cpp")))
+    for path in [os.path.join(csrc, n) for n in names] + [os.path.join(ROOT, "include", "aeon_mi355.h")]:
+        h.update(os.path.basename(path).encode())
+        h.update(open(path, "rb").read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(name):
+    """HBM bytes per launch of a kernel from a committed rocprofv3 --pmc profile
+    (profiles/traffic_<name>.json: FETCH_SIZE, WRITE_SIZE in KiB per dispatch, each scaled by what
+    the same counter reads for a plain copy of known size). Hardware counters cannot be read from
+    inside this process, so the figure is the profiler's; it is reported only while the library's
+    sources are the ones it was taken on (`csrc_digest`), otherwise as null. Returns (bytes or
+    None, the commit the profile names, whether the sources still match)."""
+    path = os.path.join(ROOT, "profiles", "traffic_%s.json" % name)
+    if not os.path.exists(path):
+        return None, None, None
     t = json.load(open(path))
-    return int(1024 * (t["fetch_size_kib_per_dispatch"] * t["fetch_scale"] +
-                       t["write_size_kib_per_dispatch"] * t["write_scale"]))
+    fresh = t.get("csrc_digest") == csrc_digest()
+    total = int(1024 * (t["fetch_size_kib_per_dispatch"] * t["fetch_scale"] +
+                        t["write_size_kib_per_dispatch"] * t["write_scale"]))
+    return (total if fresh else None), t.get("head"), fresh
 
 
 class _Calibration:
@@ -561,7 +581,25 @@ def run_prefill(layer, moe, capi, synth, torch, np, H, I, E, K_TOP, SEED, steps,
     routed_flop = 2.0 * T * K_TOP * 3 * H * I
     shared_flop = 2.0 * T * 3 * H * I
     tiles = int(np.ceil(counts / 128.0).sum()) + T // 128
+    touched = int((counts > 0).sum()) + 1
+    gu_flop = (routed_flop + shared_flop) * 2 / 3
+    gu_weight_bytes = touched * 2 * matrix_bytes(I, H)
+    traffic, traffic_head, traffic_fresh = (None, None, None)
+    if E == 256 and SCALE_GROUP == 128:
+        traffic, traffic_head, traffic_fresh = measured_traffic("config3_prefill_gate_up")
+    roofline = {
+        "kernel": "a64_grouped_kernel<gate_up> (grouped W1+W3 GEMM on fp16 MFMA, int4 dequant in "
+                  "registers, clamped SwiGLU)",
+        "bound": "mfma", "achieved": round(gu_flop / (gu_ms * 1e-3) / 1e12, 1),
+        "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+        "frac_mfma": round(gu_flop / (gu_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+        # the launch must at least stream every touched expert's two matrices once
+        "hbm_floor_bytes": int(gu_weight_bytes),
+        "frac_hbm_floor": round(gu_weight_bytes / (gu_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+        "avg_launch_ms": round(gu_ms, 4), "traffic": traffic, "traffic_head": traffic_head,
+        "traffic_sources_unchanged_since": traffic_fresh}
     return {
+        "roofline": roofline,
         "workload": "config3: prefill 2048 tokens, top-8 of %d experts, Zipf(1.1), + shared" % E,
         "ms_per_step": round(all_ms, 4),
         "tokens_per_s": round(T / (all_ms * 1e-3), 1),
@@ -987,6 +1025,9 @@ def main():
                          % (n_tok, B, len(needed) - 1, repeats, cpu_s * repeats),
                "gpu_vs_oracle_max_abs_over_peak": err}
 
+    traffic, traffic_head, traffic_fresh = (None, None, None)
+    if E == 256 and args.router_bias_scale == 1.0 and SCALE_GROUP == 128:
+        traffic, traffic_head, traffic_fresh = measured_traffic("config2_decode_b%d" % B)
     result = {
         "metric": "MoE-layer decode us/token",
         "value": round(main_run["us_per_token"], 3),
@@ -1016,13 +1057,13 @@ def main():
                      "frac": round(main_run["gate_up_gbps"] / HBM_PEAK_GBPS, 4),
                      "avg_launch_ms": round(main_run["gate_up_ms"], 4),
                      "algorithmic_bytes": int(main_run["gate_up_bytes"]),
-                     "traffic": measured_traffic(B, E, args.router_bias_scale),
-                     # hardware counters cannot be read from inside this process: the figure is
-                     # the profiler's, taken on this command and kept with its source
+                     "traffic": traffic, "traffic_head": traffic_head,
+                     "traffic_sources_unchanged_since": traffic_fresh,
                      "traffic_source": ("profiles/traffic_config2_decode_b%d.json (rocprofv3 --pmc "
                                         "FETCH_SIZE / WRITE_SIZE per dispatch of this command, scaled "
-                                        "by --calibrate-copy)" % B)
-                     if measured_traffic(B, E, args.router_bias_scale) is not None else None},
+                                        "by --calibrate-copy; null once the library's sources differ "
+                                        "from the profiled ones)" % B)
+                     if traffic_head is not None else None},
         "down_kernel": {"achieved_gbps": round(main_run["down_gbps"], 1),
                         "avg_launch_ms": round(main_run["down_ms"], 4),
                         "algorithmic_bytes": int(main_run["down_bytes"])},
