@@ -237,3 +237,56 @@ def test_config4_stacked_layers(orc, B, H, I, E, normed):
     assert torch.equal(again, final)
     unfused = moe.LayerStack(layers, mixes, norm_weights=d_norm, fused=False).step(h.dev_half(res0))
     assert torch.equal(unfused, final)
+
+
+@pytest.mark.parametrize("tokens,shared", [(1, False), (7, False), (7, True), (150, False)])
+def test_fused_reduce_post_and_next_pre_combine_equal_the_three_launches(orc, tokens, shared):
+    """aeon_moe_layer_decode_hc_post against aeon_moe_layer_decode + aeon_hc_post +
+    aeon_hc_pre_combine on the same inputs, with per-token mixes (the reference's dynamic form)
+    and with a layer that has no always-on expert (the routed sum is then added to what the
+    output rows hold): layer output, expanded residual and next layer input bit for bit, for
+    direct slots, decode segments and grouped windows."""
+    torch, h, capi, moe, synth = _setup()
+    H, I, E, k = 512, 256, 12, 4
+    pool = moe.ExpertPool(E + (1 if shared else 0), H, I)
+    assert pool.fill_synthetic(seed=71, first_expert_id=0) == 0
+    wr, bias = synth.router_weight(71, H, E), synth.router_bias(71, E)
+    layer = moe.MoeLayer(pool, E, k, shared, 7.0, h.to_dev(wr), h.to_dev(bias), score_kind=1)
+    rng = np.random.default_rng(tokens)
+
+    class Mix:
+        pass
+    this, nxt = Mix(), Mix()
+    this.post = h.to_dev(rng.uniform(0.2, 2.0, (tokens, 4)).astype(np.float32))
+    this.comb = h.to_dev(rng.uniform(0.0, 0.5, (tokens, 16)).astype(np.float32))
+    nxt.pre = h.to_dev(rng.uniform(0.1, 1.0, (tokens, 4)).astype(np.float32))
+    res = h.dev_half(synth.activations(71, 4 * tokens, H).reshape(4, tokens, H))
+    x = h.dev_half(synth.activations(72, tokens, H))
+    start = h.dev_half(synth.activations(73, tokens, H))   # what the output rows hold beforehand
+
+    out_a, ids_a, w_a = layer.decode(x, out=start.clone())
+    res_a = torch.empty_like(res)
+    capi.call("aeon_hc_post", capi.vp(out_a), C.c_long(H), capi.vp(res), C.c_long(res.stride(1)),
+              C.c_long(res.stride(0)), capi.vp(this.post), capi.vp(this.comb), 1, capi.vp(res_a),
+              tokens, H, h.stream_ptr())
+    next_a = torch.empty(tokens, H, dtype=torch.float16, device="cuda")
+    capi.call("aeon_hc_pre_combine", capi.vp(res_a), 0, C.c_long(res_a.stride(1)),
+              C.c_long(res_a.stride(0)), capi.vp(nxt.pre), 4, capi.vp(next_a), C.c_long(H), tokens, H,
+              h.stream_ptr())
+
+    res_b = torch.empty_like(res)
+    next_b = torch.empty(tokens, H, dtype=torch.float16, device="cuda")
+    out_b, ids_b, w_b = layer.decode_hc_post(x, res, res_b, this, nxt, next_b, out=start.clone())
+    torch.cuda.synchronize()
+    assert torch.equal(ids_a, ids_b) and torch.equal(w_a, w_b)
+    assert torch.equal(out_a, out_b)
+    assert torch.equal(res_a, res_b)
+    assert torch.equal(next_a, next_b)
+    # without a next layer the next-input buffer is left alone
+    untouched = torch.full_like(next_b, 3.0)
+    layer.decode_hc_post(x, res, res_b, this, None, untouched, out=start.clone())
+    torch.cuda.synchronize()
+    assert torch.all(untouched == 3.0) and torch.equal(res_a, res_b)
+    # in-place expansion is refused
+    with pytest.raises(ValueError, match="not aliased"):
+        layer.decode_hc_post(x, res, res, this, None, None, out=start.clone())
