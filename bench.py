@@ -47,17 +47,22 @@ def matrix_bytes(n, k):
 
 
 def csrc_digest():
-    """A digest of the library's sources (project-aeon_amd/csrc/*.hip, *.hpp, *.cpp and the ABI
-    header): what a committed counter profile is dated by. The GPU box runs a copy of the tree
-    without its git history, so "the kernels changed since the profile was taken" is decided by
-    content, not by commit."""
+    """A digest of the library's code (project-aeon_amd/csrc/*.hip, *.hpp, *.cpp and the ABI
+    header, comments and white space left out): what a committed counter profile is dated by. The
+    GPU box runs a copy of the tree without its git history, so "the kernels changed since the
+    profile was taken" is decided by content, not by commit; a comment edit is not a change."""
     import hashlib
+    import re
     h = hashlib.sha256()
     csrc = os.path.join(ROOT, "project-aeon_amd", "csrc")
     names = sorted(n for n in os.listdir(csrc) if n.endswith((".hip", ".hpp", ".cpp")))
     for path in [os.path.join(csrc, n) for n in names] + [os.path.join(ROOT, "include", "aeon_mi355.h")]:
+        text = open(path, encoding="utf-8").read()
+        # string literals first, so that a "//" inside one is not taken for a comment
+        text = re.sub(r'"(?:\\.|[^"\\])*"|/\*.*?\*/|//[^\n]*',
+                      lambda m: m.group(0) if m.group(0).startswith('"') else " ", text, flags=re.S)
         h.update(os.path.basename(path).encode())
-        h.update(open(path, "rb").read())
+        h.update(" ".join(text.split()).encode())
     return h.hexdigest()[:16]
 
 

@@ -103,7 +103,8 @@ __device__ __forceinline__ void grouped_run(const SegGateUpArgs& gu, const SegDo
     // Instead lanes 4q..4q+3 fetch the four pieces of position q, 64 contiguous bytes (16
     // accesses per load), rotated by q/2 so that the MFMA-order read-back -- lane (n, chunk)
     // takes unit 4n + (chunk + n/2) % 4 -- is as free of bank conflicts as a linear read
-    // (aeon_calibrate_lds_read: 2.3 ns per wave read and CU, as the linear read; 3.4 unrotated).
+    // (measured with the benchmark's LDS read-order aid: 2.3 ns per wave read and CU, as the
+    // linear read; 2.5-3.4 unrotated).
     const int load_row = lane >> 2;
     const int load_piece = ((lane & 3) - (load_row >> 1)) & 3;
     const int fragment_unit = 4 * n + ((chunk + (n >> 1)) & 3);
