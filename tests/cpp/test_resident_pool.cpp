@@ -6,6 +6,7 @@
 // directly built tables, and the loader must reject what AeonModelLoader rejects.
 #include "architecture/deepseek_v4/moe/v4_resident_expert_executor.hpp"
 #include "architecture/deepseek_v4/moe/v4_resident_expert_pool.hpp"
+#include "architecture/deepseek_v4/moe/v4_tiered_expert_executor.hpp"
 #include "backend/swizzled_w4a16/core/swizzled_expert_format.hpp"
 #include "common.hpp"
 #include "test_device.hpp"
@@ -156,6 +157,36 @@ int main() {
         }
         expect(identical, "executor over the loaded pool gives the bits of the directly built tables");
         expect(moved, "the routed experts changed the accumulator");
+    }
+    {
+        // the same container into the pinned-memory store of the two-tier executor, two experts
+        // at a time (five per layer: the last group is a short one)
+        core::V4WarmExpertStore warm(dir.string(), kHidden, kIntermediate, 2, 4096, scale_group, /*staging_experts=*/2);
+        expect(warm.layers() == kLayers && warm.experts_per_layer() == kExperts &&
+                   warm.slot_bytes() == aeon_a64_slot_bytes(kHidden, kIntermediate, scale_group),
+               "warm store: catalog shape and slot size");
+        void* d_slot = nullptr;
+        GATE_HIP(hipMalloc(&d_slot, warm.slot_bytes()));
+        aeon_a64_expert views{};
+        aeon355::throw_on_error(aeon_a64_slot_views(d_slot, kHidden, kIntermediate, scale_group, &views));
+        bool same = true;
+        for (int l = 0; l < kLayers; ++l)
+            for (int e = 0; e < kExperts; ++e) {
+                GATE_HIP(hipMemcpy(d_slot, warm.image(l, e), warm.slot_bytes(), hipMemcpyHostToDevice));
+                const void* got[6] = {views.w1_packed, views.w1_scale, views.w3_packed,
+                                      views.w3_scale, views.w2_packed, views.w2_scale};
+                const void* want[6] = {direct[l][e].w1_packed, direct[l][e].w1_scale, direct[l][e].w3_packed,
+                                       direct[l][e].w3_scale, direct[l][e].w2_packed, direct[l][e].w2_scale};
+                for (int j = 0; j < 6; ++j) {
+                    const int m = j / 2;
+                    const size_t n = j % 2 == 0 ? aeon_a64_packed_bytes(shape[m][0], shape[m][1])
+                                                : aeon_a64_scale_bytes(shape[m][0], shape[m][1], scale_group);
+                    same = same && to_host(static_cast<const uint8_t*>(got[j]), n) ==
+                                       to_host(static_cast<const uint8_t*>(want[j]), n);
+                }
+            }
+        GATE_HIP(hipFree(d_slot));
+        expect(same, "warm store: every pinned slot image equals the direct repack of its payload");
     }
     }   // scale_group
 
