@@ -49,7 +49,13 @@ struct GemvArgs {
 // HALF: a workgroup takes 8 of a tile's 16 rows (the lanes of the other 8 stay idle), so that a
 // matrix with fewer than 256 row tiles still puts a workgroup on every CU: such a launch is a
 // few microseconds long and bound by latency, not by the bytes a wave moves.
-template <int NMAT, int TOK, int WK, int SG, bool HALF>
+//
+// XLDS: the batch's activation rows are copied to LDS once per workgroup and every lane reads
+// its chunks from there. Without it a lane fetches 64 bytes per token and 128-column group from
+// memory inside the token loop, and from four tokens on those dependent fetches are a sixth of
+// the launch. (The copy comes first: with the first weights requested ahead of it the copy's
+// LDS writes wait for the weights as well -- loads return in order -- and the launch is slower.)
+template <int NMAT, int TOK, int WK, int SG, bool HALF, bool XLDS>
 __global__ __launch_bounds__(WK * 64) void a64_gemv_kernel(GemvArgs a) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -58,6 +64,15 @@ __global__ __launch_bounds__(WK * 64) void a64_gemv_kernel(GemvArgs a) {
     const int tile = HALF ? blockIdx.x >> 1 : blockIdx.x;
     const size_t tile_base = static_cast<size_t>(tile) * a.groups;
     const bool mine = !HALF || (r >> 3) == static_cast<int>(blockIdx.x & 1);
+    extern __shared__ uint4 x_lds[];  // XLDS: [tokens][groups * 16] 16-byte units
+    const int row_units = a.groups * 16;
+    if (XLDS) {
+        for (int i = threadIdx.x; i < a.tokens * row_units; i += WK * 64) {
+            const int t = i / row_units;
+            x_lds[i] = *reinterpret_cast<const uint4*>(a.x + t * a.x_stride + (i - t * row_units) * 8);
+        }
+        __syncthreads();
+    }
 
     float acc[NMAT][TOK];
 #pragma unroll
@@ -102,12 +117,20 @@ __global__ __launch_bounds__(WK * 64) void a64_gemv_kernel(GemvArgs a) {
 #pragma unroll
                 for (int t = 0; t < TOK; ++t) {
                     if (t < a.tokens) {
-                        const uint16_t* xp = a.x + t * a.x_stride + g * 128 + chunk * 8;
                         uint4 x[4];
-                        x[0] = *reinterpret_cast<const uint4*>(xp);
-                        x[1] = *reinterpret_cast<const uint4*>(xp + 32);
-                        x[2] = *reinterpret_cast<const uint4*>(xp + 64);
-                        x[3] = *reinterpret_cast<const uint4*>(xp + 96);
+                        if (XLDS) {
+                            const uint4* xp = x_lds + t * row_units + g * 16 + chunk;
+                            x[0] = xp[0];
+                            x[1] = xp[4];
+                            x[2] = xp[8];
+                            x[3] = xp[12];
+                        } else {
+                            const uint16_t* xp = a.x + t * a.x_stride + g * 128 + chunk * 8;
+                            x[0] = *reinterpret_cast<const uint4*>(xp);
+                            x[1] = *reinterpret_cast<const uint4*>(xp + 32);
+                            x[2] = *reinterpret_cast<const uint4*>(xp + 64);
+                            x[3] = *reinterpret_cast<const uint4*>(xp + 96);
+                        }
 #pragma unroll
                         for (int m = 0; m < NMAT; ++m) {
                             if (SG == 4) {
@@ -168,20 +191,49 @@ __global__ __launch_bounds__(WK * 64) void a64_gemv_kernel(GemvArgs a) {
     }
 }
 
-template <int NMAT, int TOK, int SG>
-static int launch_gemv_wk_sg(const GemvArgs& a, int wk, hipStream_t stream) {
-    const int tiles = a.N / 16;
-    if (wk >= 16 && tiles < 256 && TOK < 8) {
-        a64_gemv_kernel<NMAT, TOK, 16, SG, true><<<dim3(2 * tiles), 16 * 64, 0, stream>>>(a);
-    } else if (wk >= 16) {
-        a64_gemv_kernel<NMAT, TOK, 16, SG, false><<<dim3(tiles), 16 * 64, 0, stream>>>(a);
-    } else if (wk >= 8) {
-        a64_gemv_kernel<NMAT, TOK, 8, SG, false><<<dim3(tiles), 8 * 64, 0, stream>>>(a);
-    } else {
-        a64_gemv_kernel<NMAT, TOK, 4, SG, false><<<dim3(tiles), 4 * 64, 0, stream>>>(a);
+// From this many tokens on the activation rows are staged in LDS, where they fit beside the
+// 16 KiB of partial sums (one or two tokens gain nothing from it: measured).
+constexpr int kGemvXldsMinTokens = 4;
+constexpr size_t kGemvXldsMaxBytes = 128 * 1024;
+
+template <int NMAT, int TOK, int WK, int SG, bool HALF, bool XLDS>
+static int launch_gemv_one(const GemvArgs& a, int blocks, size_t x_bytes, hipStream_t stream) {
+    auto* kernel = a64_gemv_kernel<NMAT, TOK, WK, SG, HALF, XLDS>;
+    if (XLDS) {
+        // more dynamic LDS than the default limit has to be asked for, once per kernel
+        static bool raised = false;
+        if (!raised) {
+            AEON_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         static_cast<int>(kGemvXldsMaxBytes)));
+            raised = true;
+        }
     }
+    kernel<<<dim3(blocks), WK * 64, XLDS ? x_bytes : 0, stream>>>(a);
     AEON_LAUNCH_CHECK();
     return AEON_OK;
+}
+
+template <int NMAT, int TOK, int SG, bool XLDS>
+static int launch_gemv_wk_sg_x(const GemvArgs& a, int wk, size_t x_bytes, hipStream_t stream) {
+    const int tiles = a.N / 16;
+    if (wk >= 16 && tiles < 256 && TOK < 8) {
+        return launch_gemv_one<NMAT, TOK, 16, SG, true, XLDS>(a, 2 * tiles, x_bytes, stream);
+    } else if (wk >= 16) {
+        return launch_gemv_one<NMAT, TOK, 16, SG, false, XLDS>(a, tiles, x_bytes, stream);
+    } else if (wk >= 8) {
+        return launch_gemv_one<NMAT, TOK, 8, SG, false, XLDS>(a, tiles, x_bytes, stream);
+    }
+    return launch_gemv_one<NMAT, TOK, 4, SG, false, XLDS>(a, tiles, x_bytes, stream);
+}
+
+template <int NMAT, int TOK, int SG>
+static int launch_gemv_wk_sg(const GemvArgs& a, int wk, hipStream_t stream) {
+    const size_t x_bytes = static_cast<size_t>(a.tokens) * a.groups * 256;
+    if constexpr (TOK >= kGemvXldsMinTokens) {
+        if (x_bytes <= kGemvXldsMaxBytes) return launch_gemv_wk_sg_x<NMAT, TOK, SG, true>(a, wk, x_bytes, stream);
+    }
+    return launch_gemv_wk_sg_x<NMAT, TOK, SG, false>(a, wk, x_bytes, stream);
 }
 
 template <int NMAT, int TOK>
