@@ -15,6 +15,7 @@
 //     in fp32 to the per-group MFMA result, so dequantisation stays exact.
 #include "expert_a64.hpp"
 
+#include <atomic>
 
 namespace aeon355 {
 
@@ -200,13 +201,16 @@ template <int NMAT, int TOK, int WK, int SG, bool HALF, bool XLDS>
 static int launch_gemv_one(const GemvArgs& a, int blocks, size_t x_bytes, hipStream_t stream) {
     auto* kernel = a64_gemv_kernel<NMAT, TOK, WK, SG, HALF, XLDS>;
     if (XLDS) {
-        // more dynamic LDS than the default limit has to be asked for, once per kernel
-        static bool raised = false;
-        if (!raised) {
+        // more dynamic LDS than the default limit has to be asked for, once per kernel and device
+        static std::atomic<uint64_t> raised{0};
+        int device = 0;
+        AEON_HIP(hipGetDevice(&device));
+        const uint64_t bit = 1ull << (device & 63);
+        if (device >= 64 || (raised.load(std::memory_order_relaxed) & bit) == 0) {
             AEON_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                          hipFuncAttributeMaxDynamicSharedMemorySize,
                                          static_cast<int>(kGemvXldsMaxBytes)));
-            raised = true;
+            raised.fetch_or(bit, std::memory_order_relaxed);
         }
     }
     kernel<<<dim3(blocks), WK * 64, XLDS ? x_bytes : 0, stream>>>(a);
