@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the routed-expert hot path on one MI355X.
 
-A "step" is one full MoE-layer decode (BASELINE config 2: fp32 router 7168x256 -> sigmoid+bias
+A "step" is one full MoE-layer decode (benchmark config 2: fp32 router 7168x256 -> sigmoid+bias
 top-8 -> 256 int4 W4A16 experts + 1 always-on shared expert -> fixed-order weighted sum) over
 one batch of synthetic tokens, with every expert resident in HBM in the wave64 packing and all
 inputs already on the device when the timed region starts.
@@ -286,7 +286,7 @@ def run_dropin(capi, moe, torch, np):
     ms = a.elapsed_time(b) / 320
     res["token_trio"] = {"ms_per_token": round(ms, 4),
                          "weights_gbps": round(K * expert_bytes / ms / 1e6, 1)}
-    # the single GEMV and dual GEMV entry points: the reference's shape and BASELINE config 0's,
+    # the single GEMV and dual GEMV entry points: the reference's shape and benchmark config 0's,
     # 64 launches on different matrices captured into one graph (a launch is shorter than a call)
     res["gemv"] = []
     for cols in (H, 7168):
@@ -548,7 +548,7 @@ def run_window_classes(layer, moe, capi, synth, torch, np, H, I, E, K_TOP, SEED)
 
 
 def run_prefill(layer, moe, capi, synth, torch, np, H, I, E, K_TOP, SEED, steps, warmup):
-    """BASELINE config 3: 2048 tokens, top-8 of 256 experts with Zipf(1.1) popularity, through the
+    """benchmark config 3: 2048 tokens, top-8 of 256 experts with Zipf(1.1) popularity, through the
     permutation -> grouped gate+up GEMM + SwiGLU -> grouped W2 GEMM -> fixed-order reduce path.
     FLOPs are the algorithmic 2*positions*3*H*I (routed draws + the shared expert's tokens)."""
     T = 2048
@@ -624,7 +624,7 @@ def run_prefill(layer, moe, capi, synth, torch, np, H, I, E, K_TOP, SEED, steps,
 
 def run_other_configs(pool, layer, moe, capi, synth, torch, np, H, I, E, K_TOP, LIMIT, SEED, wr, bias,
                       B, steps):
-    """Configs 0, 1 and 4 of BASELINE.json. Configs 0/1 rotate through every resident expert
+    """Configs 0, 1 and 4 of the benchmark definition. Configs 0/1 rotate through every resident expert
     (5.8 GB) so no launch finds its weights in the 256 MB Infinity Cache."""
     def timed(fn, reps):
         """Mean time of one call. The calls are a few microseconds long, shorter than a launch
@@ -743,7 +743,7 @@ def run_other_configs(pool, layer, moe, capi, synth, torch, np, H, I, E, K_TOP, 
                 "frac_of_peak": round(bytes4 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                 "finite": bool(torch.isfinite(r.float()).all())}
 
-    # as BASELINE writes it: nothing normalises the residual between the layers, so its scale grows,
+    # as the benchmark definition writes it: nothing normalises the residual between the layers, so its scale grows,
     # the sigmoid scores of layers 2-4 saturate and the bias alone picks their experts
     res["config4_stack"] = run_stack(moe.LayerStack(layers, mixes, fused=True))
     res["config4_stack"]["launches_per_layer"] = "router logits, top-k, permutation, gate/up, down, " \
@@ -775,7 +775,7 @@ def main():
                          "the default run reports in `other_configs`")
     ap.add_argument("--all-configs", dest="all_configs", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--router-bias-scale", type=float, default=1.0,
-                    help="scale of the per-expert router bias in the headline leg (1 = BASELINE's "
+                    help="scale of the per-expert router bias in the headline leg (1 = the benchmark definition's "
                          "N(0, 0.1); 0 = no bias, the spread routing)")
     ap.add_argument("--no-unbiased", action="store_true",
                     help="skip the second decode leg (router bias removed); a kernel profile of the "

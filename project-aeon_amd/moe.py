@@ -319,7 +319,7 @@ class DynamicHyperConnection:
 
 
 class LayerStack:
-    """BASELINE config 4: stacked MoE layers with the hyper-connection residual mix between them.
+    """benchmark config 4: stacked MoE layers with the hyper-connection residual mix between them.
     Per layer: x = pre-combine(residual); [x = RMSNorm(x) * norm_weight]; y = MoE(x);
     residual = post-mix(y, residual). `norm_weights`: None = no norm (the configuration as
     written); a list with one entry per layer, each a device fp16 [hidden] weight or None for the

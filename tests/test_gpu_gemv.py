@@ -54,7 +54,7 @@ def test_swizzled_gemv_reference_fixture(orc, N, K, cfg):
 
 
 def test_config0_single_gemv_both_layouts(orc):
-    """BASELINE config 0: x [1x7168] ~N(0,1), W int4 [7168->2048], group-128 scales, seed 0."""
+    """benchmark config 0: x [1x7168] ~N(0,1), W int4 [7168->2048], group-128 scales, seed 0."""
     torch, h, capi = _setup()
     from project_aeon_amd import synth
     N, K = 2048, 7168
@@ -239,7 +239,7 @@ def test_swizzled_expert_trio_reference_shapes(orc, experts):
 @pytest.mark.parametrize("use_mfma", [0, 1])
 @pytest.mark.parametrize("tokens", [1, 4, 8])
 def test_config1_one_expert_decode(orc, tokens, use_mfma, scale_group):
-    """BASELINE config 1: one routed expert, batch 1/4/8, H=7168, I=2048, clamp 7, output scaled
+    """benchmark config 1: one routed expert, batch 1/4/8, H=7168, I=2048, clamp 7, output scaled
     by a router weight in (0,1]; with one scale per 128 columns (the config) and with a scale
     of its own per 32 columns (the `.aeon` format's grouping)."""
     torch, h, capi = _setup()

@@ -162,7 +162,7 @@ def test_config4_stacked_layers(orc, B, H, I, E, normed):
     """Four MoE layers with independent seeded weights and the HC mix between them. Each layer is
     checked against the oracle on the device's own input to that layer and the device's routed
     ids (the way a composed gate isolates one stage from the rounding of the ones before it).
-    The third case is BASELINE config 4 as written: 4 x (256 + 1) resident experts (23 GB), batch
+    The third case is benchmark config 4 as written: 4 x (256 + 1) resident experts (23 GB), batch
     64; there the oracle takes three tokens of every layer and its experts' payloads come back
     from the device generator. `normed` puts the FFN RMSNorm (seeded weight) between the
     pre-combine and the router/experts, where the reference's layer body has it

@@ -1,5 +1,5 @@
 """GPU parity for the device-resident MoE layer: synthetic experts generated and re-swizzled on
-the device, router logits / top-k / permutation, and the full decode step of BASELINE config 2
+the device, router logits / top-k / permutation, and the full decode step of benchmark config 2
 against the oracle."""
 import ctypes as C
 
@@ -283,7 +283,7 @@ def _oracle_layer_streamed(orc, make_expert, x, ids, weights, shared, limit):
 
 @pytest.mark.parametrize("B", [1, 8, 32, 64])
 def test_config2_moe_layer_decode_reduced_experts(orc, B):
-    """BASELINE config 2 at full hidden/intermediate with a 24-expert layer (so the oracle can
+    """benchmark config 2 at full hidden/intermediate with a 24-expert layer (so the oracle can
     regenerate every expert): fp32 router [7168 x E], sigmoid + bias, top-8, renormalised, one
     always-on shared expert, int4 group-128 experts."""
     torch, h, capi, moe, synth = _setup()
@@ -391,7 +391,7 @@ def test_group32_scales_on_the_resident_path(orc, H, I, E, k, T, shared):
 
 
 def test_config2_full_size_sampled(orc):
-    """BASELINE config 2 as written: batch 64, top-8 of 256 experts + the always-on one, fp32
+    """benchmark config 2 as written: batch 64, top-8 of 256 experts + the always-on one, fp32
     router with sigmoid scores and bias, H=7168, I=2048. The oracle covers a sample of tokens
     (ids bit-exact on the device's logits for all of them); the rest is covered by properties
     that hold at any size: a token's output does not depend on the other tokens of the batch
@@ -680,7 +680,7 @@ def test_prefill_window_bodies_at_every_live_count(orc):
 
 
 def test_config3_prefill_full_size_sampled(orc):
-    """BASELINE config 3 at full size: 2048 tokens, top-8 of 256 experts with Zipf(1.1)
+    """benchmark config 3 at full size: 2048 tokens, top-8 of 256 experts with Zipf(1.1)
     popularity, H=7168, I=2048, + shared expert. The oracle covers a sample of tokens; the rest
     is covered by parity with the decode path on 64 tokens and by a token-permutation property
     (reversing the token order permutes the output rows and nothing else)."""
