@@ -107,6 +107,31 @@ def test_a64_gemv_and_dual(orc, tokens, N, K, matrix, scale_group):
     assert torch.equal(single, oa)
 
 
+@pytest.mark.parametrize("tokens,N,K", [(5, 2048, 7168), (8, 7168, 2048), (8, 64, 16384)])
+def test_a64_gemv_batch_rows_staged_or_fetched(orc, tokens, N, K):
+    """From four tokens on the batch's activation rows are copied to LDS once per workgroup where
+    they fit (8 x 7168 halves do, 8 x 16384 do not and are fetched per lane as before): both
+    forms against the oracle, and a batch whose rows sit in a wider buffer gives the bits of the
+    packed one."""
+    torch, h, capi = _setup()
+    from project_aeon_amd import synth
+    m = h.synth_matrix(5, 1, 0, N, K, 128)
+    x = synth.activations(11, tokens, K)
+    want = orc.swizzled_matvec(m.swz_packed, m.swz_scale, N, K, *m.cfg, x.astype(np.float64))
+    pa, sa = h.dev_u32(m.a64_packed), h.dev_u16(m.a64_scale)
+    packed = h.dev_half(x)
+    wide = torch.full((tokens, K + 72), 3.0, dtype=torch.float16, device="cuda")
+    wide[:, :K] = packed
+    outs = []
+    for buf, pitch in ((packed, K), (wide, K + 72)):
+        out = torch.zeros(tokens, N, dtype=torch.float16, device="cuda")
+        capi.call("aeon_a64_gemv", capi.vp(buf), pitch, capi.vp(pa), capi.vp(sa), 128, capi.vp(out), N,
+                  tokens, N, K, h.stream_ptr())
+        outs.append(out)
+    assert h.rel_err(outs[0].cpu().numpy(), want) <= TOL
+    assert torch.equal(outs[0], outs[1])
+
+
 def test_swizzled_dual_equals_two_singles(orc):
     torch, h, capi = _setup()
     from project_aeon_amd import synth
