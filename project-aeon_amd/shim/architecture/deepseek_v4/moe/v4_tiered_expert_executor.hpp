@@ -292,11 +292,12 @@ public:
         }
         CHECK_HIP(hipMalloc(&workspace_, workspace_bytes_));
         CHECK_HIP(hipMalloc(reinterpret_cast<void**>(&d_ids_), sizeof(int32_t) * max_tokens * widest_top_k));
-        CHECK_HIP(hipHostMalloc(reinterpret_cast<void**>(&h_ids_), sizeof(int32_t) * max_tokens * widest_top_k,
+        ids_per_dispatch_ = static_cast<size_t>(max_tokens) * widest_top_k;
+        CHECK_HIP(hipHostMalloc(reinterpret_cast<void**>(&h_ids_), sizeof(int32_t) * ids_per_dispatch_ * kIdRing,
                                 hipHostMallocDefault));
         CHECK_HIP(hipEventCreateWithFlags(&compute_mark_, hipEventDisableTiming));
         CHECK_HIP(hipEventCreateWithFlags(&uploads_done_, hipEventDisableTiming));
-        CHECK_HIP(hipEventCreateWithFlags(&ids_consumed_, hipEventDisableTiming));
+        for (hipEvent_t& e : ids_consumed_) CHECK_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
     }
 
     ~V4HbmTieredExpertExecutor() override {
@@ -304,7 +305,7 @@ public:
         (void)hipStreamSynchronize(streams_.compute);
         (void)hipEventDestroy(compute_mark_);
         (void)hipEventDestroy(uploads_done_);
-        (void)hipEventDestroy(ids_consumed_);
+        for (hipEvent_t e : ids_consumed_) (void)hipEventDestroy(e);
         (void)hipFree(workspace_);
         (void)hipFree(d_ids_);
         (void)hipFree(d_tables_);
@@ -395,13 +396,16 @@ public:
         awaiting_uploads_ = awaiting_uploads_ || marked;
 
         // the per-token path needs the ids on the device; a chunk passes its own device ids.
-        // The pinned staging row may still be read by the copy of the dispatch before.
-        if (ids_in_flight_) CHECK_HIP(hipEventSynchronize(ids_consumed_));
-        std::memcpy(h_ids_, flat.data(), flat.size() * sizeof(int32_t));
-        CHECK_HIP(hipMemcpyAsync(d_ids_, h_ids_, flat.size() * sizeof(int32_t), hipMemcpyHostToDevice,
+        // They are staged in a ring of pinned rows: the copy out of a row may still be queued
+        // behind earlier layers' kernels, and the host only waits for it when the ring comes
+        // round to that row again.
+        const size_t turn = dispatches_++ % kIdRing;
+        if (dispatches_ > kIdRing) CHECK_HIP(hipEventSynchronize(ids_consumed_[turn]));
+        int32_t* staged = h_ids_ + turn * ids_per_dispatch_;
+        std::memcpy(staged, flat.data(), flat.size() * sizeof(int32_t));
+        CHECK_HIP(hipMemcpyAsync(d_ids_, staged, flat.size() * sizeof(int32_t), hipMemcpyHostToDevice,
                                  streams_.compute));
-        CHECK_HIP(hipEventRecord(ids_consumed_, streams_.compute));
-        ids_in_flight_ = true;
+        CHECK_HIP(hipEventRecord(ids_consumed_[turn], streams_.compute));
 
         current_layer_ = static_cast<int64_t>(layer_id);
         first_position_ = first_position;
@@ -512,9 +516,12 @@ private:
     size_t workspace_bytes_{0};
     int32_t* d_ids_{nullptr};
     int32_t* h_ids_{nullptr};
-    hipEvent_t compute_mark_{nullptr}, uploads_done_{nullptr}, ids_consumed_{nullptr};
+    static constexpr size_t kIdRing = 16;
+    size_t ids_per_dispatch_{0};
+    uint64_t dispatches_{0};
+    hipEvent_t compute_mark_{nullptr}, uploads_done_{nullptr};
+    hipEvent_t ids_consumed_[kIdRing] = {};
     bool awaiting_uploads_{false};
-    bool ids_in_flight_{false};
 
     int64_t current_layer_{-1};
     uint32_t first_position_{0};

@@ -255,6 +255,49 @@ int main() {
     } catch (const std::invalid_argument&) { few_slots = true; }
     expect(no_slots && few_slots, "a pool with no slots, or fewer than one token routes to, is refused at construction");
 
+    // --- what the protocol costs when nothing misses: the same three layers again and again ----
+    {
+        core::V4HotExpertSlots roomy(warm, 20);
+        core::V4HbmTieredExpertExecutor executor(warm, roomy, layers, 16, streams);
+        std::vector<int32_t> ids = {0, 1, 2, 3, 4, 5};
+        std::vector<float> w(kSlots, 0.2f);
+        float* d_w = to_device(w);
+        half* out = to_device(std::vector<half>(shared.begin(), shared.begin() + row));
+        auto walk = [&](core::V4RoutedExpertExecutor& e, core::ExpertLeaseHolder* holder, int tokens) {
+            for (int t = 0; t < tokens; ++t) {
+                for (int l = 0; l < kLayers; ++l) {
+                    e.on_routing_ready(l, 1000 + t, ids, w);
+                    e.accumulate_routed(l, 1000 + t, d_x, d_w, out);
+                    e.on_routed_consumed(l, 1000 + t);
+                }
+                if (holder != nullptr) holder->release_leases();
+            }
+            GATE_HIP(hipStreamSynchronize(streams.compute));
+        };
+        auto timed = [&](core::V4RoutedExpertExecutor& e, core::ExpertLeaseHolder* holder) {
+            walk(e, holder, 20);
+            hipEvent_t begin, end;
+            GATE_HIP(hipEventCreate(&begin));
+            GATE_HIP(hipEventCreate(&end));
+            GATE_HIP(hipEventRecord(begin, streams.compute));
+            walk(e, holder, 200);
+            GATE_HIP(hipEventRecord(end, streams.compute));
+            GATE_HIP(hipEventSynchronize(end));
+            float ms = 0;
+            GATE_HIP(hipEventElapsedTime(&ms, begin, end));
+            return ms * 1000.0f / (200 * kLayers);
+        };
+        const float us_tiered = timed(executor, &executor);
+        const float us_resident = timed(resident, nullptr);
+        const core::V4TierCounters c = executor.counters();
+        std::printf("  all resident in the pool: %.1f us per layer step through the two-tier executor, %.1f us through the "
+                    "all-resident one (%llu uploads in %llu dispatches)\n", us_tiered, us_resident,
+                    static_cast<unsigned long long>(c.warm_uploads),
+                    static_cast<unsigned long long>((c.hot_hits + c.warm_uploads) / kSlots));
+        expect(c.warm_uploads == static_cast<uint64_t>(kLayers) * kSlots && c.forced_drains == 0,
+               "a working set that fits is uploaded once and then only found");
+    }
+
     // --- what a miss costs: one slot image over the host link -------------------------------
     {
         hipEvent_t begin, end;
