@@ -187,6 +187,48 @@ int main() {
             }
         GATE_HIP(hipFree(d_slot));
         expect(same, "warm store: every pinned slot image equals the direct repack of its payload");
+
+        // container -> warm store -> three HBM slots -> two-tier executor, against the executor
+        // over the directly built tables: five experts a layer through three slots, so the walk
+        // evicts, and every token of every layer has to come out with the same bits
+        core::V4TierStreams streams;
+        GATE_HIP(hipStreamCreateWithFlags(&streams.compute, hipStreamNonBlocking));
+        GATE_HIP(hipStreamCreateWithFlags(&streams.upload, hipStreamNonBlocking));
+        std::vector<aeon_moe_layer> routing(kLayers), from_direct(kLayers);
+        for (int l = 0; l < kLayers; ++l) {
+            routing[l] = aeon_moe_layer{kHidden, kIntermediate, kExperts, kSlots, 0, 7.0f, AEON_ROUTER_SCORE_SIGMOID,
+                                        1.0f, 1, nullptr, nullptr, nullptr, scale_group};
+            from_direct[l] = routing[l];
+            from_direct[l].d_experts = to_device(direct[l]);
+        }
+        core::V4HotExpertSlots hot(warm, 3);
+        core::V4HbmTieredExpertExecutor tiered(warm, hot, routing, 16, streams);
+        core::V4ResidentExpertExecutor control(from_direct, 16, streams.compute);
+        SplitMix rng{0x1207E8C0ull};
+        std::vector<half> x(static_cast<size_t>(kTokens) * kHidden), shared(x.size());
+        for (half& v : x) v = __float2half(static_cast<float>(rng.uniform() - 0.5));
+        for (half& v : shared) v = __float2half(static_cast<float>(rng.uniform() - 0.5));
+        half* d_x = to_device(x);
+        half* out_t = to_device(shared);
+        half* out_c = to_device(shared);
+        for (int t = 0; t < kTokens; ++t) {
+            for (int l = 0; l < kLayers; ++l) {
+                const std::vector<int32_t> ids = {(2 * t + l) % kExperts, (2 * t + l + 3) % kExperts};
+                const std::vector<float> w = {0.7f, 0.3f};
+                float* d_w = to_device(w);
+                tiered.on_routing_ready(l, t, ids, w);
+                tiered.accumulate_routed(l, t, d_x + static_cast<size_t>(t) * kHidden, d_w,
+                                         out_t + static_cast<size_t>(t) * kHidden);
+                control.on_routing_ready(l, t, ids, w);
+                control.accumulate_routed(l, t, d_x + static_cast<size_t>(t) * kHidden, d_w,
+                                          out_c + static_cast<size_t>(t) * kHidden);
+            }
+            GATE_HIP(hipStreamSynchronize(streams.compute));
+            tiered.release_leases();
+        }
+        const std::vector<half> rt = to_host(out_t, x.size()), rc = to_host(out_c, x.size());
+        expect(std::memcmp(rt.data(), rc.data(), rt.size() * sizeof(half)) == 0 && tiered.counters().evictions > 0,
+               "two-tier executor over the container, three slots for ten experts: the bits of the direct tables");
     }
     }   // scale_group
 
